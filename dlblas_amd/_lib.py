@@ -1,0 +1,173 @@
+"""ctypes binding of libdlblas_fp8_gemm.so (the C ABI declared in include/dlblas_fp8_gemm.h).
+
+The library is the only implementation: when it has not been built, every op raises ImportError.  There is no
+PyTorch or CPU fallback.  The calling convention (``c_void_p(tensor.data_ptr())`` operands, the stream handle as
+``c_void_p``) is the one the reference uses for its native code, tests/kernels/cutlass/test_fp8_convert.py:8-39.
+"""
+import ctypes
+import os
+import threading
+
+import torch
+
+from ._build import LIB_PATH
+
+ABI_VERSION = 1
+OUT_BF16, OUT_F32 = 0, 1
+WS_COUNTER_BYTES = 65536
+WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
+
+ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_BAD_STRIDE, ERR_BAD_DTYPE, ERR_WORKSPACE, ERR_ALIGNMENT, ERR_LAUNCH = \
+    -1, -2, -3, -4, -5, -6, -7
+
+_c_i64, _c_i32, _c_vp, _c_sz = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.c_size_t
+
+# name -> (restype, argtypes); must list every symbol include/dlblas_fp8_gemm.h declares
+SYMBOLS = {
+    'dlb_abi_version': (ctypes.c_int, []),
+    'dlb_last_error': (ctypes.c_char_p, []),
+    'dlb_fp8_gemm_workspace_bytes': (_c_sz, [_c_i64, _c_i64, _c_i64]),
+    'dlb_fp8_gemm': (ctypes.c_int, [_c_vp] * 5 + [_c_i64] * 5 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
+    'dlb_fp8_gemm_grouped_contiguous':
+    (ctypes.c_int, [_c_vp] * 6 + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 2 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
+    'dlb_fp8_gemm_grouped_masked':
+    (ctypes.c_int, [_c_vp] * 6 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 3 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
+    'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
+    'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
+}
+
+_lock = threading.Lock()
+_lib = None
+_workspaces = {}
+
+
+def library_path() -> str:
+    return os.environ.get('DLBLAS_AMD_LIB', LIB_PATH)
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once; ImportError (never a silent fallback) when it is missing or stale."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = library_path()
+        if not os.path.exists(path):
+            raise ImportError(f'{path} has not been built; run `python -m dlblas_amd._build` '
+                              '(needs hipcc) - there is no fallback implementation')
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as exc:
+            raise ImportError(f'cannot load {path}: {exc}') from exc
+        for name, (restype, argtypes) in SYMBOLS.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError:
+                raise ImportError(f'{path} does not export {name}; rebuild it') from None
+            fn.restype, fn.argtypes = restype, argtypes
+        if lib.dlb_abi_version() != ABI_VERSION:
+            raise ImportError(f'{path} has ABI version {lib.dlb_abi_version()}, expected {ABI_VERSION}; rebuild it')
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().dlb_last_error().decode()
+
+
+def check(rc: int) -> None:
+    """Map a negative return code of the C ABI to a Python exception."""
+    if rc == 0:
+        return
+    msg = f'dlblas fp8_gemm error {rc}: {last_error()}'
+    if rc in (ERR_BAD_SHAPE, ERR_BAD_STRIDE, ERR_BAD_DTYPE, ERR_NULL_POINTER, ERR_ALIGNMENT):
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+def workspace(device: torch.device, stream_handle: int) -> torch.Tensor:
+    """Zero-initialised scratch buffer, one per (device, stream): calls on one stream never overlap."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_handle)
+    buf = _workspaces.get(key)
+    if buf is None:
+        buf = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def variant_names():
+    lib = load()
+    names, i = [], 0
+    while True:
+        name = lib.dlb_fp8_gemm_variant_name(i)
+        if name is None:
+            return names
+        names.append(name.decode())
+        i += 1
+
+
+def force_variant(name_or_id) -> None:
+    """Pin the kernel variant used by later calls from this thread (None or -1: back to the heuristic)."""
+    lib = load()
+    if name_or_id is None:
+        name_or_id = -1
+    if isinstance(name_or_id, str):
+        name_or_id = variant_names().index(name_or_id)
+    check(lib.dlb_fp8_gemm_force_variant(int(name_or_id)))
+
+
+def out_code(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return OUT_BF16
+    if dtype == torch.float32:
+        return OUT_F32
+    raise ValueError(f'fp8_gemm output dtype must be bfloat16 or float32, got {dtype}')
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
+
+
+def _stream_and_ws(t: torch.Tensor):
+    stream = torch.cuda.current_stream(t.device).cuda_stream
+    ws = workspace(t.device, stream)
+    return stream, ws
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError('dlblas fp8_gemm runs on the GPU only; got a tensor on ' + str(t.device))
+
+
+def gemm_dense(a, b, a_s, b_s, c, M, N, K, as_sm, as_sk):
+    _require_gpu(a, b, a_s, b_s, c)
+    lib = load()
+    with torch.cuda.device(a.device):
+        stream, ws = _stream_and_ws(a)
+        check(lib.dlb_fp8_gemm(_ptr(a), _ptr(b), _ptr(a_s), _ptr(b_s), _ptr(c), M, N, K, as_sm, as_sk,
+                               out_code(c.dtype), _ptr(ws), ws.numel(), ctypes.c_void_p(stream)))
+
+
+def gemm_contiguous(a, b, a_s, b_s, c, m_indices, M_sum, N, K, G, as_sm, as_sk):
+    _require_gpu(a, b, a_s, b_s, c, m_indices)
+    lib = load()
+    with torch.cuda.device(a.device):
+        stream, ws = _stream_and_ws(a)
+        check(
+            lib.dlb_fp8_gemm_grouped_contiguous(_ptr(a), _ptr(b), _ptr(a_s), _ptr(b_s), _ptr(c), _ptr(m_indices),
+                                                M_sum, N, K, G, as_sm, as_sk, out_code(c.dtype), _ptr(ws),
+                                                ws.numel(), ctypes.c_void_p(stream)))
+
+
+def gemm_masked(a, b, a_s, b_s, c, masked_m, expected_m, M_max, N, K, G, as_sg, as_sm, as_sk):
+    _require_gpu(a, b, a_s, b_s, c, masked_m)
+    lib = load()
+    with torch.cuda.device(a.device):
+        stream, ws = _stream_and_ws(a)
+        check(
+            lib.dlb_fp8_gemm_grouped_masked(_ptr(a), _ptr(b), _ptr(a_s), _ptr(b_s), _ptr(c), _ptr(masked_m),
+                                            int(expected_m), M_max, N, K, G, as_sg, as_sm, as_sk,
+                                            out_code(c.dtype), _ptr(ws), ws.numel(), ctypes.c_void_p(stream)))

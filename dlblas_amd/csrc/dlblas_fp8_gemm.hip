@@ -1,0 +1,411 @@
+// C ABI of the gfx950 FP8 block-scaled GEMM library: argument validation, kernel selection, launches.
+// The declarations and the contract of every entry point are in include/dlblas_fp8_gemm.h.
+#include "../../include/dlblas_fp8_gemm.h"
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "fp8_gemm_common.h"
+#include "fp8_gemm_skinny.h"
+#include "fp8_gemm_tiled.h"
+
+namespace dlb {
+
+// ---------------------------------------------------------------------------------------------------------
+// Exact path for shapes the MFMA kernels do not take (K not a multiple of 16): one thread per output
+// element, e4m3 decoded in software, fp32 FMA chain per 128 block, scales applied as in
+// dlblas/kernels/fp8_gemm.py:55.
+// ---------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) fp8_gemm_exact_kernel(const Args p) {
+  const int n = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (m >= p.M || n >= p.N) return;
+  const uint8_t* a_row = p.a + static_cast<int64_t>(m) * p.K;
+  const uint8_t* b_row = p.b + static_cast<int64_t>(n) * p.K;
+  const float* as_row = p.a_s + static_cast<int64_t>(m) * p.as_sm;
+  const float* bs_row = p.b_s + static_cast<int64_t>(n / kScaleBlock) * p.kblocks;
+  float acc = 0.f;
+  for (int kb = 0; kb < p.kblocks; ++kb) {
+    const int k1 = min(p.K, (kb + 1) * kScaleBlock);
+    float dot = 0.f;
+    for (int k = kb * kScaleBlock; k < k1; ++k) dot = fmaf(e4m3_to_f32(a_row[k]), e4m3_to_f32(b_row[k]), dot);
+    acc += dot * as_row[static_cast<int64_t>(kb) * p.as_sk] * bs_row[kb];
+  }
+  if (p.out_f32)
+    static_cast<float*>(p.c)[static_cast<int64_t>(m) * p.N + n] = acc;
+  else
+    static_cast<__bf16*>(p.c)[static_cast<int64_t>(m) * p.N + n] = static_cast<__bf16>(acc);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------------------
+namespace {
+
+thread_local char g_err[256] = "";
+thread_local int g_forced_variant = -1;
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+enum Variant : int {
+  kVarExact = 0,
+  kVarTile128x128,
+  kVarTile64x128,
+  kVarTile128x64,
+  kVarSkinny16,
+  kVarSkinny32,
+  kVarCount
+};
+
+const char* const kVariantNames[kVarCount] = {
+    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32",
+};
+
+typedef TileCfg<128, 128, 2, 2> Tile128x128;
+typedef TileCfg<64, 128, 2, 2> Tile64x128;
+typedef TileCfg<128, 64, 2, 2> Tile128x64;
+typedef SkinnyCfg<1, 4> Skinny16;
+typedef SkinnyCfg<2, 4> Skinny32;
+
+constexpr int kMaxDevices = 64;
+
+int device_cu_count(int* dev_out) {
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  *dev_out = dev;
+  if (dev < 0 || dev >= kMaxDevices) return 256;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    cached[dev].store(cus, std::memory_order_relaxed);
+  }
+  return cus;
+}
+
+// Raise a kernel's dynamic LDS limit once per (kernel, device).
+template <class Kernel>
+hipError_t ensure_lds(Kernel kernel, int bytes, int dev, std::atomic<unsigned long long>* done_mask) {
+  if (bytes <= 48 * 1024) return hipSuccess;
+  const unsigned long long bit = 1ull << (dev & 63);
+  if (done_mask->load(std::memory_order_acquire) & bit) return hipSuccess;
+  const hipError_t e =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done_mask->fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
+template <class Cfg, int MODE>
+hipError_t launch_tiled(const Args& args, int grid, int dev, hipStream_t stream) {
+  static std::atomic<unsigned long long> lds_done{0};
+  auto kernel = fp8_gemm_tiled_kernel<Cfg, MODE>;
+  hipError_t e = ensure_lds(kernel, Cfg::LDS_BYTES, dev, &lds_done);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+  return hipGetLastError();
+}
+
+template <class Cfg>
+hipError_t launch_tiled_mode(int mode, const Args& args, int grid, int dev, hipStream_t stream) {
+  switch (mode) {
+    case kDense:
+      return launch_tiled<Cfg, kDense>(args, grid, dev, stream);
+    case kContiguous:
+      return launch_tiled<Cfg, kContiguous>(args, grid, dev, stream);
+    default:
+      return launch_tiled<Cfg, kMasked>(args, grid, dev, stream);
+  }
+}
+
+template <class Cfg>
+hipError_t launch_skinny(const Args& args, hipStream_t stream) {
+  hipLaunchKernelGGL(fp8_gemm_skinny_kernel<Cfg>, dim3(args.tiles_n * args.splitk), dim3(Cfg::NT), 0, stream, args);
+  return hipGetLastError();
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+struct Plan {
+  int variant;
+  int bm, bn;
+  int splitk;
+};
+
+void tile_dims(int variant, int* bm, int* bn) {
+  switch (variant) {
+    case kVarTile64x128:
+      *bm = 64, *bn = 128;
+      break;
+    case kVarTile128x64:
+      *bm = 128, *bn = 64;
+      break;
+    case kVarSkinny16:
+      *bm = 16, *bn = 16;
+      break;
+    case kVarSkinny32:
+      *bm = 32, *bn = 16;
+      break;
+    default:
+      *bm = 128, *bn = 128;
+  }
+}
+
+bool is_skinny(int v) { return v == kVarSkinny16 || v == kVarSkinny32; }
+
+// Largest split count (<= limit) whose slices still hold `min_kb` K blocks each.
+int pick_splitk(int64_t units, int kblocks, int cus, int waves_per_unit, int min_kb, int limit) {
+  // aim for about four waves per SIMD over the whole chip
+  const int64_t want_waves = static_cast<int64_t>(cus) * 16;
+  int s = static_cast<int>(ceil_div(want_waves, units * waves_per_unit));
+  s = s < 1 ? 1 : s;
+  if (s > limit) s = limit;
+  if (s > kblocks / min_kb) s = kblocks / min_kb;
+  return s < 1 ? 1 : s;
+}
+
+Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes) {
+  Plan pl{kVarTile128x128, 128, 128, 1};
+  const int kblocks = static_cast<int>(ceil_div(K, kScaleBlock));
+  int v = g_forced_variant;
+  if (v < 0) {
+    if (K % 16 != 0)
+      v = kVarExact;
+    else if (mode == kDense && M <= 16)
+      v = kVarSkinny16;
+    else if (mode == kDense && M <= 32)
+      v = kVarSkinny32;
+    else if (M <= 64 && mode != kContiguous)
+      v = kVarTile64x128;
+    else
+      v = kVarTile128x128;
+  }
+  if (K % 16 != 0) v = kVarExact;
+  if (is_skinny(v) && (mode != kDense || M > (v == kVarSkinny16 ? 16 : 32))) v = kVarTile128x128;
+  if (v == kVarExact && mode != kDense) v = kVarTile128x128;
+  pl.variant = v;
+  tile_dims(v, &pl.bm, &pl.bn);
+  if (mode != kDense || v == kVarExact || kblocks < 2) return pl;
+
+  const int64_t tiles_n = ceil_div(N, pl.bn);
+  const size_t avail = ws_bytes > DLB_WS_COUNTER_BYTES ? ws_bytes - DLB_WS_COUNTER_BYTES : 0;
+  if (is_skinny(v)) {
+    if (tiles_n > DLB_WS_COUNTER_BYTES / 4) return pl;
+    int s = pick_splitk(tiles_n, kblocks, cus, 4, 4, 16);
+    const size_t per_split = static_cast<size_t>(tiles_n) * (pl.bm / 16) * 256 * sizeof(float);
+    while (s > 1 && per_split * s > avail) --s;
+    pl.splitk = s;
+  } else {
+    const int64_t tiles = ceil_div(M, pl.bm) * tiles_n;
+    if (tiles > DLB_WS_COUNTER_BYTES / 4 || tiles * 2 > cus) return pl;
+    int s = pick_splitk(tiles, kblocks, cus, 16, 2, 16);
+    const size_t per_split = static_cast<size_t>(tiles) * pl.bm * pl.bn * sizeof(float);
+    while (s > 1 && per_split * s > avail) --s;
+    pl.splitk = s;
+  }
+  return pl;
+}
+
+struct Problem {
+  int mode;
+  const void *a, *b;
+  const float *a_s, *b_s;
+  void* c;
+  const int32_t* gidx;
+  int64_t rows;  // dense: M, contiguous: M_sum, masked: M_max
+  int64_t N, K;
+  int G;
+  int64_t as_sg, as_sm, as_sk;
+  int out_dtype;
+  void* ws;
+  size_t ws_bytes;
+  hipStream_t stream;
+};
+
+bool misaligned(const void* ptr, size_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) != 0; }
+
+int run(const Problem& pr) {
+  g_err[0] = '\0';
+  if (pr.out_dtype != DLB_OUT_BF16 && pr.out_dtype != DLB_OUT_F32)
+    return fail(DLB_ERR_BAD_DTYPE, "out_dtype %d is neither DLB_OUT_BF16 nor DLB_OUT_F32", pr.out_dtype);
+  if (pr.rows < 0 || pr.N < 0 || pr.K < 0)
+    return fail(DLB_ERR_BAD_SHAPE, "negative dimension (rows=%lld N=%lld K=%lld)", (long long)pr.rows,
+                (long long)pr.N, (long long)pr.K);
+  const int64_t lim = (1ll << 31) - 1024;
+  if (pr.rows > lim || pr.N > lim || pr.K > lim)
+    return fail(DLB_ERR_BAD_SHAPE, "dimension beyond 2^31 (rows=%lld N=%lld K=%lld)", (long long)pr.rows,
+                (long long)pr.N, (long long)pr.K);
+  if (pr.mode != kDense && pr.G < 0) return fail(DLB_ERR_BAD_SHAPE, "negative group count %d", pr.G);
+  const int64_t groups = pr.mode == kDense ? 1 : pr.G;
+  if (pr.rows == 0 || pr.N == 0 || groups == 0) return DLB_OK;
+  if (!pr.c) return fail(DLB_ERR_NULL_POINTER, "c is NULL");
+  if (pr.mode != kDense && !pr.gidx)
+    return fail(DLB_ERR_NULL_POINTER, "%s is NULL", pr.mode == kContiguous ? "m_indices" : "masked_m");
+  if (pr.K > 0 && (!pr.a || !pr.b || !pr.a_s || !pr.b_s))
+    return fail(DLB_ERR_NULL_POINTER, "a, b, a_s or b_s is NULL");
+  if (pr.mode != kDense && pr.K % 16 != 0)
+    return fail(DLB_ERR_BAD_SHAPE, "grouped GEMM needs K %% 16 == 0 (K=%lld)", (long long)pr.K);
+  const int64_t kblocks = ceil_div(pr.K, kScaleBlock);
+  if (pr.K > 0) {
+    if (pr.as_sm < 0 || pr.as_sk < 0 || pr.as_sg < 0)
+      return fail(DLB_ERR_BAD_STRIDE, "negative a_s stride");
+    if (pr.rows > 1 && pr.as_sm == 0) return fail(DLB_ERR_BAD_STRIDE, "a_s row stride is 0 for %lld rows", (long long)pr.rows);
+    if (kblocks > 1 && pr.as_sk == 0) return fail(DLB_ERR_BAD_STRIDE, "a_s K-block stride is 0 for %lld blocks", (long long)kblocks);
+    if (pr.mode == kMasked && pr.G > 1 && pr.as_sg == 0) return fail(DLB_ERR_BAD_STRIDE, "a_s group stride is 0");
+  }
+  const bool mfma_path = pr.K % 16 == 0;
+  if (mfma_path && pr.K > 0 && (misaligned(pr.a, 16) || misaligned(pr.b, 16)))
+    return fail(DLB_ERR_ALIGNMENT, "a and b must be 16-byte aligned");
+  if (misaligned(pr.c, 2) || misaligned(pr.a_s, 4) || misaligned(pr.b_s, 4))
+    return fail(DLB_ERR_ALIGNMENT, "c / a_s / b_s are not aligned to their element size");
+
+  int dev = 0;
+  const int cus = device_cu_count(&dev);
+  if (cus < 0) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
+
+  Plan pl = make_plan(pr.mode, pr.rows, pr.N, pr.K, cus, pr.ws ? pr.ws_bytes : 0);
+  if (pl.splitk > 1) {
+    if (!pr.ws || pr.ws_bytes < DLB_WS_COUNTER_BYTES) pl.splitk = 1;
+    if (misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
+  }
+
+  Args ar;
+  memset(&ar, 0, sizeof(ar));
+  ar.a = static_cast<const uint8_t*>(pr.a);
+  ar.b = static_cast<const uint8_t*>(pr.b);
+  ar.a_s = pr.a_s;
+  ar.b_s = pr.b_s;
+  ar.c = pr.c;
+  ar.gidx = pr.gidx;
+  ar.M = static_cast<int>(pr.rows);
+  ar.N = static_cast<int>(pr.N);
+  ar.K = static_cast<int>(pr.K);
+  ar.G = pr.mode == kDense ? 1 : pr.G;
+  ar.kblocks = static_cast<int>(kblocks);
+  ar.nblocks = static_cast<int>(ceil_div(pr.N, kScaleBlock));
+  ar.as_sm = pr.as_sm;
+  ar.as_sk = pr.as_sk;
+  ar.as_gs = pr.as_sg;
+  ar.a_gs = pr.rows * pr.K;
+  ar.c_gs = pr.rows * pr.N;
+  ar.b_gs = pr.N * pr.K;
+  ar.bs_gs = static_cast<int64_t>(ar.nblocks) * kblocks;
+  ar.tiles_m = static_cast<int>(ceil_div(pr.rows, pl.bm));
+  ar.tiles_n = static_cast<int>(ceil_div(pr.N, pl.bn));
+  ar.splitk = pl.splitk;
+  ar.kb_per_split = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, pl.splitk));
+  ar.splitk = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, ar.kb_per_split));  // no empty splits
+  ar.group_m = 8;
+  ar.out_f32 = pr.out_dtype == DLB_OUT_F32;
+  const size_t esz = ar.out_f32 ? 4 : 2;
+  ar.vec_store = (pr.N % 4 == 0) && !misaligned(pr.c, 4 * esz);
+  if (pr.ws && pr.ws_bytes >= DLB_WS_COUNTER_BYTES) {
+    ar.ctr = static_cast<uint32_t*>(pr.ws);
+    ar.ws = reinterpret_cast<float*>(static_cast<char*>(pr.ws) + DLB_WS_COUNTER_BYTES);
+  }
+
+  hipError_t e = hipSuccess;
+  const int64_t tiles = static_cast<int64_t>(ar.tiles_m) * ar.tiles_n * ar.splitk;
+  switch (pl.variant) {
+    case kVarExact: {
+      if (pr.mode != kDense) return fail(DLB_ERR_BAD_SHAPE, "exact path is dense only");
+      const dim3 grid(static_cast<unsigned>(ceil_div(pr.N, 64)), static_cast<unsigned>(ceil_div(pr.rows, 4)));
+      hipLaunchKernelGGL(fp8_gemm_exact_kernel, grid, dim3(256), 0, pr.stream, ar);
+      e = hipGetLastError();
+      break;
+    }
+    case kVarSkinny16:
+      e = launch_skinny<Skinny16>(ar, pr.stream);
+      break;
+    case kVarSkinny32:
+      e = launch_skinny<Skinny32>(ar, pr.stream);
+      break;
+    default: {
+      int64_t grid = tiles;
+      if (pr.mode == kMasked) {
+        // the real tile count is only known on the device; cover the worst case with a resident-sized grid
+        const int64_t worst = static_cast<int64_t>(ar.tiles_m) * ar.tiles_n * pr.G;
+        grid = worst < static_cast<int64_t>(cus) * 4 ? worst : static_cast<int64_t>(cus) * 4;
+      }
+      if (grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)grid);
+      const int g = static_cast<int>(grid);
+      if (pl.variant == kVarTile64x128)
+        e = launch_tiled_mode<Tile64x128>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarTile128x64)
+        e = launch_tiled_mode<Tile128x64>(pr.mode, ar, g, dev, pr.stream);
+      else
+        e = launch_tiled_mode<Tile128x128>(pr.mode, ar, g, dev, pr.stream);
+    }
+  }
+  if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return DLB_OK;
+}
+
+}  // namespace
+}  // namespace dlb
+
+// ---------------------------------------------------------------------------------------------------------
+// extern "C" surface
+// ---------------------------------------------------------------------------------------------------------
+extern "C" {
+
+int dlb_abi_version(void) { return DLB_ABI_VERSION; }
+
+const char* dlb_last_error(void) { return dlb::g_err; }
+
+size_t dlb_fp8_gemm_workspace_bytes(int64_t rows, int64_t N, int64_t K) {
+  (void)K;
+  if (rows <= 0 || N <= 0) return DLB_WS_COUNTER_BYTES;
+  // Split-K is only used while the un-split grid cannot fill the chip, i.e. for at most ~256 tiles of
+  // 128 x 128 fp32 partials times at most 16 splits; small-M problems need far less.
+  const int64_t tiles = dlb::ceil_div(rows, 64) * dlb::ceil_div(N, 64);
+  const int64_t capped = tiles < 1024 ? tiles : 1024;
+  return DLB_WS_COUNTER_BYTES + static_cast<size_t>(capped) * 64 * 64 * sizeof(float) * 16;
+}
+
+int dlb_fp8_gemm(const void* a, const void* b, const float* a_s, const float* b_s, void* c, int64_t M, int64_t N,
+                 int64_t K, int64_t as_stride_m, int64_t as_stride_k, int out_dtype, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+  dlb::Problem pr{dlb::kDense, a, b, a_s, b_s, c, nullptr, M, N, K, 1, 0, as_stride_m, as_stride_k, out_dtype,
+                  workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  return dlb::run(pr);
+}
+
+int dlb_fp8_gemm_grouped_contiguous(const void* a, const void* b, const float* a_s, const float* b_s, void* c,
+                                    const int32_t* m_indices, int64_t M_sum, int64_t N, int64_t K, int32_t G,
+                                    int64_t as_stride_m, int64_t as_stride_k, int out_dtype, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  dlb::Problem pr{dlb::kContiguous, a, b, a_s, b_s, c, m_indices, M_sum, N, K, G, 0, as_stride_m, as_stride_k,
+                  out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  return dlb::run(pr);
+}
+
+int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, const float* b_s, void* c,
+                                const int32_t* masked_m, int32_t expected_m, int64_t M_max, int64_t N, int64_t K,
+                                int32_t G, int64_t as_stride_g, int64_t as_stride_m, int64_t as_stride_k,
+                                int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  (void)expected_m;
+  dlb::Problem pr{dlb::kMasked, a, b, a_s, b_s, c, masked_m, M_max, N, K, G, as_stride_g, as_stride_m, as_stride_k,
+                  out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  return dlb::run(pr);
+}
+
+int dlb_fp8_gemm_force_variant(int variant) {
+  if (variant >= dlb::kVarCount) return dlb::fail(DLB_ERR_BAD_SHAPE, "unknown kernel variant %d", variant);
+  dlb::g_forced_variant = variant < 0 ? -1 : variant;
+  return DLB_OK;
+}
+
+const char* dlb_fp8_gemm_variant_name(int variant) {
+  if (variant < 0 || variant >= dlb::kVarCount) return nullptr;
+  return dlb::kVariantNames[variant];
+}
+
+}  // extern "C"

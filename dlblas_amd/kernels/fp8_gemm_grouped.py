@@ -1,0 +1,157 @@
+"""Grouped FP8 block-scaled GEMMs for MoE experts: expert-contiguous rows and masked fixed-capacity buffers.
+
+The reference does not implement these; it forwards to the third-party ``deep_gemm`` package
+(dlblas/kernels/fused_moe_v3.py:235-245 and dlblas/layers/moe/ep_moe.py:180-197).  The functions here take the
+positional arguments those call sites pass, under both generations of deep_gemm names the call sites probe,
+write ``out`` in place and return None.
+"""
+from typing import Sequence
+
+import torch
+
+from .. import _lib
+from ..utils import SymVar, Tensor, register_dlblas_op
+
+BLOCK = 128
+
+
+def _unpack(pair: Sequence[torch.Tensor], what: str):
+    if not isinstance(pair, (tuple, list)) or len(pair) != 2:
+        raise TypeError(f'{what} must be a (tensor, scales) pair')
+    return pair[0], pair[1]
+
+
+def _check_common(a, a_s, w, w_s, out):
+    for name, t, dt in (('a', a, torch.float8_e4m3fn), ('w', w, torch.float8_e4m3fn), ('a_s', a_s, torch.float32),
+                        ('w_s', w_s, torch.float32)):
+        if t.dtype != dt:
+            raise TypeError(f'{name} must be {dt}, got {t.dtype}')
+    if out.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f'out must be bfloat16 or float32, got {out.dtype}')
+    assert a.is_contiguous() and w.is_contiguous() and out.is_contiguous(), 'Input tensors must be contiguous'
+    assert w_s.is_contiguous(), 'Scaling factor tensors must be contiguous'
+    if w.dim() != 3:
+        raise ValueError(f'weights must be [G, N, K], got {tuple(w.shape)}')
+    G, N, K = w.shape
+    if K % 16 != 0:
+        raise ValueError(f'grouped fp8 gemm needs K % 16 == 0, got K={K}')
+    if tuple(w_s.shape) != (G, -(-N // BLOCK), -(-K // BLOCK)):
+        raise ValueError(f'w_s must be [{G}, {-(-N // BLOCK)}, {-(-K // BLOCK)}], got {tuple(w_s.shape)}')
+    return G, N, K
+
+
+@torch.library.custom_op('dlblas::fp8_gemm_grouped_contiguous', mutates_args=('out', ), device_types='cuda')
+def grouped_contiguous_op(a: torch.Tensor, a_s: torch.Tensor, w: torch.Tensor, w_s: torch.Tensor,
+                          out: torch.Tensor, m_indices: torch.Tensor) -> None:
+    G, N, K = w.shape
+    _lib.gemm_contiguous(a, w, a_s, w_s, out, m_indices, a.size(0), N, K, G, a_s.stride(0), a_s.stride(1))
+
+
+@torch.library.custom_op('dlblas::fp8_gemm_grouped_masked', mutates_args=('out', ), device_types='cuda')
+def grouped_masked_op(a: torch.Tensor, a_s: torch.Tensor, w: torch.Tensor, w_s: torch.Tensor, out: torch.Tensor,
+                      masked_m: torch.Tensor, expected_m: int) -> None:
+    G, N, K = w.shape
+    _lib.gemm_masked(a, w, a_s, w_s, out, masked_m, expected_m, a.size(1), N, K, G, a_s.stride(0), a_s.stride(1),
+                     a_s.stride(2))
+
+
+def fp8_gemm_grouped_contiguous(a, a_s, w, w_s, out, m_indices):
+    """``out[r] = (a[r] * a_s[r]) @ (w[g] * w_s[g]).T`` with ``g = m_indices[r]``; rows of an expert are
+    contiguous, every expert's span is a multiple of 128 rows, a 128-row block whose first index is negative
+    is skipped.  ``a_s`` may be any strided 2-D view (the reference passes a column-major one,
+    dlblas/kernels/quant_dequant.py:65-83)."""
+    G, N, K = _check_common(a, a_s, w, w_s, out)
+    if a.dim() != 2 or a.size(1) != K:
+        raise ValueError(f'a must be [M_sum, {K}], got {tuple(a.shape)}')
+    M_sum = a.size(0)
+    if tuple(a_s.shape) != (M_sum, -(-K // BLOCK)):
+        raise ValueError(f'a_s must be [{M_sum}, {-(-K // BLOCK)}], got {tuple(a_s.shape)}')
+    if tuple(out.shape) != (M_sum, N):
+        raise ValueError(f'out must be [{M_sum}, {N}], got {tuple(out.shape)}')
+    if m_indices.dtype != torch.int32 or tuple(m_indices.shape) != (M_sum, ) or not m_indices.is_contiguous():
+        raise ValueError('m_indices must be a contiguous int32 vector with one entry per row of a')
+    grouped_contiguous_op(a, a_s, w, w_s, out, m_indices)
+
+
+def fp8_gemm_grouped_masked(a, a_s, w, w_s, out, masked_m, expected_m=0):
+    """For every expert g, rows ``[0, masked_m[g])`` of ``out[g]`` get ``(a[g] * a_s[g]) @ (w[g] * w_s[g]).T``;
+    the other rows of ``out`` are left untouched and the matching rows of ``a`` are never used."""
+    G, N, K = _check_common(a, a_s, w, w_s, out)
+    if a.dim() != 3 or a.size(0) != G or a.size(2) != K:
+        raise ValueError(f'a must be [{G}, M_max, {K}], got {tuple(a.shape)}')
+    M_max = a.size(1)
+    if tuple(a_s.shape) != (G, M_max, -(-K // BLOCK)):
+        raise ValueError(f'a_s must be [{G}, {M_max}, {-(-K // BLOCK)}], got {tuple(a_s.shape)}')
+    if tuple(out.shape) != (G, M_max, N):
+        raise ValueError(f'out must be [{G}, {M_max}, {N}], got {tuple(out.shape)}')
+    if masked_m.dtype != torch.int32 or tuple(masked_m.shape) != (G, ) or not masked_m.is_contiguous():
+        raise ValueError('masked_m must be a contiguous int32 vector with one entry per expert')
+    grouped_masked_op(a, a_s, w, w_s, out, masked_m, int(expected_m))
+
+
+# --- deep_gemm-compatible positional entry points (what the reference's shims call) --------------------------
+
+
+def m_grouped_fp8_gemm_nt_contiguous(input_tuple, w_tuple, out, m_indices, *unused, **unused_kw):
+    a, a_s = _unpack(input_tuple, 'input_tuple')
+    w, w_s = _unpack(w_tuple, 'w_tuple')
+    fp8_gemm_grouped_contiguous(a, a_s, w, w_s, out, m_indices)
+
+
+def m_grouped_fp8_gemm_nt_masked(input_tuple, w_tuple, out, masked_m, expected_m, *unused, **unused_kw):
+    a, a_s = _unpack(input_tuple, 'input_tuple')
+    w, w_s = _unpack(w_tuple, 'w_tuple')
+    fp8_gemm_grouped_masked(a, a_s, w, w_s, out, masked_m, expected_m)
+
+
+m_grouped_gemm_fp8_fp8_bf16_nt_contiguous = m_grouped_fp8_gemm_nt_contiguous
+m_grouped_gemm_fp8_fp8_bf16_nt_masked = m_grouped_fp8_gemm_nt_masked
+
+
+def _event_bench(fn, warmup=3, rep=10) -> float:
+    for _ in range(warmup):
+        fn()
+    times = []
+    for _ in range(rep):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        stop.record()
+        stop.synchronize()
+        times.append(start.elapsed_time(stop))
+    times.sort()
+    return times[len(times) // 2]
+
+
+def _bench_contiguous(a, a_s, w, w_s, out, m_indices):
+    return _event_bench(lambda: fp8_gemm_grouped_contiguous(a, a_s, w, w_s, out, m_indices))
+
+
+def _bench_masked(a, a_s, w, w_s, out, masked_m, expected_m=0):
+    return _event_bench(lambda: fp8_gemm_grouped_masked(a, a_s, w, w_s, out, masked_m, expected_m))
+
+
+def _register():
+    f8, f32, i32, dev = torch.float8_e4m3fn, torch.float32, torch.int32, 'cuda'
+    g, m, n, k, kb, nb = (SymVar(s) for s in ('g', 'm', 'n', 'k', 'kb', 'nb'))
+    for out_dtype in (torch.bfloat16, torch.float32):
+        register_dlblas_op('fp8_gemm_grouped_contiguous', None, (
+            Tensor((m, k), dtype=f8, device=dev),
+            Tensor((m, kb), dtype=f32, device=dev),
+            Tensor((g, n, k), dtype=f8, device=dev),
+            Tensor((g, nb, kb), dtype=f32, device=dev),
+            Tensor((m, n), dtype=out_dtype, device=dev),
+            Tensor((m, ), dtype=i32, device=dev),
+        ), fp8_gemm_grouped_contiguous, _bench_contiguous, fp8_gemm_grouped_contiguous)
+        register_dlblas_op('fp8_gemm_grouped_masked', None, (
+            Tensor((g, m, k), dtype=f8, device=dev),
+            Tensor((g, m, kb), dtype=f32, device=dev),
+            Tensor((g, n, k), dtype=f8, device=dev),
+            Tensor((g, nb, kb), dtype=f32, device=dev),
+            Tensor((g, m, n), dtype=out_dtype, device=dev),
+            Tensor((g, ), dtype=i32, device=dev),
+            torch.SymInt,
+        ), fp8_gemm_grouped_masked, _bench_masked, fp8_gemm_grouped_masked)
+
+
+_register()

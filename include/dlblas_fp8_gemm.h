@@ -1,0 +1,157 @@
+/*
+ * dlblas_fp8_gemm.h -- C ABI of the MI355X (gfx950) FP8 block-scaled GEMM library.
+ *
+ * All three GEMM entry points compute, for every output element,
+ *
+ *     C[m, n] = sum_kb ( sum_{k in block kb} A[m, k] * B[n, k] ) * a_s[m, kb] * b_s[n / 128, kb]
+ *
+ * with A, B in OCP float8 e4m3fn, one fp32 activation scale per (row, 128-wide K block),
+ * one fp32 weight scale per (128 x 128) block of B, fp32 accumulation, and a single cast to the
+ * output type at the end.  "NT" layout: A is [M, K] and B is [N, K], both K-contiguous.
+ *
+ * Conventions shared by every function here
+ *   - plain pointers and sizes only; every pointer is a DEVICE pointer unless stated otherwise;
+ *   - the library never allocates, frees or synchronises; work is enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL = the null stream) and the call returns at once;
+ *   - return value 0 = enqueued, negative = rejected (see DLB_ERR_*), nothing was enqueued;
+ *     dlb_last_error() gives a thread-local human-readable reason for the last failure;
+ *   - no C++ exception ever crosses this boundary;
+ *   - `workspace` is caller-owned device memory of at least dlb_fp8_gemm_workspace_bytes()
+ *     bytes.  Its first DLB_WS_COUNTER_BYTES bytes are tile counters: they must be ZERO the
+ *     first time the buffer is used and are left zero by every call, so one buffer can be
+ *     reused by any number of calls that do not overlap in time.  Two calls that may run
+ *     concurrently (different streams) need separate workspaces.
+ *
+ * Reference interfaces these replace (paths relative to the DLBlas source tree):
+ *   - dlb_fp8_gemm                     : dlblas/kernels/fp8_gemm.py:15-65 (kernel) and :68-89 (host wrapper)
+ *   - dlb_fp8_gemm_grouped_contiguous  : deep_gemm.m_grouped_fp8_gemm_nt_contiguous as called from
+ *                                        dlblas/kernels/fused_moe_v3.py:235-245
+ *   - dlb_fp8_gemm_grouped_masked      : deep_gemm.m_grouped_fp8_gemm_nt_masked as called from
+ *                                        dlblas/layers/moe/ep_moe.py:180-197
+ *   - the ctypes calling convention (void* data pointers, void* stream) follows the reference's only
+ *     native entry point, dlblas/kernels/cutlass/fp8_convert.cu:8 and its loader
+ *     tests/kernels/cutlass/test_fp8_convert.py:8-39.
+ */
+#ifndef DLBLAS_FP8_GEMM_H_
+#define DLBLAS_FP8_GEMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DLB_ABI_VERSION 1
+
+/* output element type of C */
+#define DLB_OUT_BF16 0
+#define DLB_OUT_F32 1
+
+/* error codes (all negative) */
+#define DLB_OK 0
+#define DLB_ERR_NULL_POINTER (-1)   /* a required pointer is NULL                                  */
+#define DLB_ERR_BAD_SHAPE (-2)      /* a dimension is negative / too large / violates a constraint */
+#define DLB_ERR_BAD_STRIDE (-3)     /* a stride cannot address the stated shape                    */
+#define DLB_ERR_BAD_DTYPE (-4)      /* out_dtype is not DLB_OUT_BF16 / DLB_OUT_F32                  */
+#define DLB_ERR_WORKSPACE (-5)      /* workspace is NULL or smaller than required                  */
+#define DLB_ERR_ALIGNMENT (-6)      /* a pointer is not 16-byte aligned where the kernels need it  */
+#define DLB_ERR_LAUNCH (-7)         /* the HIP runtime refused the launch                          */
+
+/* bytes at the head of every workspace that hold self-resetting tile counters */
+#define DLB_WS_COUNTER_BYTES 65536
+
+/* Version of this ABI (DLB_ABI_VERSION of the library that was loaded). */
+int dlb_abi_version(void);
+
+/* Thread-local description of the last failure on the calling thread ("" if none). */
+const char* dlb_last_error(void);
+
+/*
+ * Upper bound of the workspace any of the three GEMM entry points can need for a problem with
+ * `rows` activation rows in total (M, M_sum, or G * M_max), N outputs per row and contraction
+ * length K.  Never fails; returns at least DLB_WS_COUNTER_BYTES.
+ */
+size_t dlb_fp8_gemm_workspace_bytes(int64_t rows, int64_t N, int64_t K);
+
+/*
+ * Dense block-scaled GEMM.   Replaces fp8_gemm_kernel / fp8_gemm (dlblas/kernels/fp8_gemm.py:15-89).
+ *
+ *   a    [M, K]                     e4m3fn, row-major, row stride K
+ *   b    [N, K]                     e4m3fn, row-major, row stride K
+ *   a_s  [M, ceil(K/128)]           fp32, element (m, kb) at a_s[m * as_stride_m + kb * as_stride_k]
+ *   b_s  [ceil(N/128), ceil(K/128)] fp32, row-major
+ *   c    [M, N]                     bf16 or fp32 (out_dtype), row-major, row stride N
+ *
+ * M, N, K >= 0 (M == 0 or N == 0 enqueues nothing; K == 0 stores zeros).  Any M, N, K are accepted;
+ * K % 16 == 0 takes the MFMA path, other K a slower exact path.
+ */
+int dlb_fp8_gemm(const void* a, const void* b, const float* a_s, const float* b_s, void* c,
+                 int64_t M, int64_t N, int64_t K,
+                 int64_t as_stride_m, int64_t as_stride_k,
+                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Grouped GEMM, expert-contiguous rows.  Replaces deep_gemm.m_grouped_fp8_gemm_nt_contiguous
+ * (call site dlblas/kernels/fused_moe_v3.py:235-245, buffers built at :262-308).
+ *
+ *   a         [M_sum, K]                      e4m3fn, row stride K
+ *   a_s       [M_sum, ceil(K/128)]            fp32, addressed through as_stride_m / as_stride_k
+ *                                             (the reference hands over a column-major view)
+ *   b         [G, N, K]                       e4m3fn, contiguous
+ *   b_s       [G, ceil(N/128), ceil(K/128)]   fp32, contiguous
+ *   c         [M_sum, N]                      bf16 or fp32, row stride N, caller allocated
+ *   m_indices [M_sum]                         int32: expert of each row.  Rows of one expert are
+ *                                             contiguous and every expert's span is a multiple of 128
+ *                                             rows, so the expert is read once per aligned 128-row
+ *                                             block (from its first row); a negative value skips the
+ *                                             block and leaves its rows of c untouched.
+ *
+ * M_sum need not be a multiple of 128 (the last block may be short).  K % 16 == 0 is required.
+ */
+int dlb_fp8_gemm_grouped_contiguous(const void* a, const void* b, const float* a_s, const float* b_s,
+                                    void* c, const int32_t* m_indices,
+                                    int64_t M_sum, int64_t N, int64_t K, int32_t G,
+                                    int64_t as_stride_m, int64_t as_stride_k,
+                                    int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Grouped GEMM, fixed-capacity buffers with a valid-row count per expert.  Replaces
+ * deep_gemm.m_grouped_fp8_gemm_nt_masked (call site dlblas/layers/moe/ep_moe.py:180-197,
+ * buffers built at :199-261).
+ *
+ *   a         [G, M_max, K]                   e4m3fn, contiguous
+ *   a_s       [G, M_max, ceil(K/128)]         fp32, element (g, m, kb) at
+ *                                             a_s[g * as_stride_g + m * as_stride_m + kb * as_stride_k]
+ *   b         [G, N, K]                       e4m3fn, contiguous
+ *   b_s       [G, ceil(N/128), ceil(K/128)]   fp32, contiguous
+ *   c         [G, M_max, N]                   bf16 or fp32, contiguous, caller allocated
+ *   masked_m  [G]                             int32 on the device: rows [0, masked_m[g]) of expert g
+ *                                             are computed; rows at or beyond it are neither read
+ *                                             into a valid result nor written.  Values are clamped
+ *                                             to [0, M_max].
+ *   expected_m                                scheduling hint only (typical masked_m); <= 0 = unknown
+ *
+ * The tile schedule is built on the device from masked_m: no host synchronisation and no tiles
+ * for empty row ranges.  K % 16 == 0 is required.
+ */
+int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, const float* b_s,
+                                void* c, const int32_t* masked_m, int32_t expected_m,
+                                int64_t M_max, int64_t N, int64_t K, int32_t G,
+                                int64_t as_stride_g, int64_t as_stride_m, int64_t as_stride_k,
+                                int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Tuning / test hook: force the kernel variant the next calls FROM THIS THREAD use.
+ * variant < 0 restores the built-in shape heuristic.  Returns DLB_ERR_BAD_SHAPE for an unknown id.
+ * Variant ids are listed by dlb_fp8_gemm_variant_name().
+ */
+int dlb_fp8_gemm_force_variant(int variant);
+
+/* Name of kernel variant `variant`, or NULL beyond the last one. */
+const char* dlb_fp8_gemm_variant_name(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DLBLAS_FP8_GEMM_H_ */

@@ -1,0 +1,201 @@
+"""GPU parity of the HIP kernels (through the Python entry points -> C ABI) against the CPU oracle."""
+import pytest
+import torch
+
+import helpers
+from oracle import fp8_block_gemm as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def dev():
+    import dlblas_amd  # noqa: F401
+    from dlblas_amd import _lib
+    _lib.load()
+    return torch.device('cuda:0')
+
+
+def _run_dense(dev, a_q, a_s, b_q, b_s, dtype=torch.bfloat16, variant=None):
+    from dlblas_amd import _lib
+    from dlblas_amd.kernels.fp8_gemm import fp8_gemm
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(dtype)
+    try:
+        _lib.force_variant(variant)
+        out = fp8_gemm(a_q.to(dev), b_q.to(dev), a_s.to(dev), b_s.to(dev))
+        torch.cuda.synchronize()
+    finally:
+        _lib.force_variant(None)
+        torch.set_default_dtype(prev)
+    return out
+
+
+DENSE_SHAPES = [
+    (64, 512, 1024),      # the reference's CPU-runnable configuration
+    (512, 512, 512),      # the shape of tests/kernels/test_fp8_gemm.py
+    (1, 7168, 2048), (16, 7168, 2048), (64, 7168, 2048), (128, 7168, 2048),
+    (1, 2112, 7168), (16, 2112, 7168), (64, 2112, 7168), (128, 2112, 7168),
+    (300, 2112, 1536),    # ragged M and N tiles
+    (129, 130, 384),      # N not a multiple of 4: scalar stores
+    (33, 200, 400),       # K tail (400 = 3 * 128 + 16)
+    (17, 64, 200),        # K not a multiple of 16: exact path
+]
+
+
+@pytest.mark.parametrize('M,N,K', DENSE_SHAPES)
+def test_dense_bf16_matches_oracle(dev, M, N, K):
+    print(f'case dense bf16 M={M} N={N} K={K}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    out = _run_dense(dev, a_q, a_s, b_q, b_s)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (M, N)
+    helpers.tolerance_check(out, ref, f'dense {M}x{N}x{K}')
+
+
+@pytest.mark.parametrize('variant', ['tile128x128', 'tile64x128', 'tile128x64', 'skinny16', 'skinny32', 'exact'])
+@pytest.mark.parametrize('M,N,K', [(16, 512, 1024), (30, 200, 400), (200, 392, 2048)])
+def test_every_variant(dev, variant, M, N, K):
+    print(f'case variant={variant} M={M} N={N} K={K}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=7)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    out = _run_dense(dev, a_q, a_s, b_q, b_s, variant=variant)
+    helpers.tolerance_check(out, ref, f'{variant} {M}x{N}x{K}')
+
+
+def test_dense_f32_reference_test_construction(dev):
+    """The reference's own test: randn e4m3 operands, randn (signed) scales, fp32 out, atol 1e-1
+    (tests/kernels/test_fp8_gemm.py:8-31,70-72)."""
+    print('case dense f32 reference construction', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_raw(512, 512, 512)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    out = _run_dense(dev, a_q, a_s, b_q, b_s, dtype=torch.float32)
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out.cpu(), ref, atol=1e-1, rtol=0)
+    helpers.tolerance_check(out, ref, 'reference construction')
+
+
+def test_dense_exact_small_integers(dev):
+    """Operands holding small integers and unit scales: every partial sum is an integer below 2^24, so the fp32
+    result is exact whatever the summation order - bit-exact comparison."""
+    print('case dense exact integers', flush=True)
+    g = helpers.gen(3)
+    M, N, K = 48, 272, 640
+    a = torch.randint(-4, 5, (M, K), generator=g).float()
+    b = torch.randint(-4, 5, (N, K), generator=g).float()
+    a_q, b_q = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
+    a_s, b_s = torch.ones(M, 5), torch.ones(3, 5)
+    out = _run_dense(dev, a_q, a_s, b_q, b_s, dtype=torch.float32)
+    assert torch.equal(out.cpu(), a @ b.t())
+
+
+def test_leading_dims_are_flattened(dev):
+    print('case leading dims', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(6 * 5, 256, 256, seed=11)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    out = _run_dense(dev, a_q.reshape(6, 5, 256), a_s.reshape(6, 5, 2), b_q, b_s)
+    assert tuple(out.shape) == (6, 5, 256)
+    helpers.tolerance_check(out.reshape(30, 256), ref, 'leading dims')
+
+
+def test_contiguity_asserts(dev):
+    from dlblas_amd.kernels.fp8_gemm import fp8_gemm
+    a_q, a_s, b_q, b_s = (t.to(dev) for t in helpers.make_dense(32, 256, 256))
+    with pytest.raises(AssertionError, match='Input tensors must be contiguous'):
+        fp8_gemm(a_q.t().contiguous().t(), b_q, a_s, b_s)
+    with pytest.raises(AssertionError, match='Scaling factor tensors must be contiguous'):
+        fp8_gemm(a_q, b_q, a_s.t().contiguous().t(), b_s)
+
+
+def test_repeat_calls_are_deterministic(dev):
+    """Split-K partials are added in split order by whichever workgroup arrives last: bit-identical reruns."""
+    print('case determinism', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(16, 2112, 7168, seed=5)
+    outs = [_run_dense(dev, a_q, a_s, b_q, b_s) for _ in range(3)]
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    a_q, a_s, b_q, b_s = helpers.make_dense(128, 1024, 4096, seed=5)
+    outs = [_run_dense(dev, a_q, a_s, b_q, b_s) for _ in range(3)]
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+# ----------------------------------------------------------------------------------------------------------------
+# grouped
+# ----------------------------------------------------------------------------------------------------------------
+def _make_grouped_weights(G, N, K, seed):
+    g = helpers.gen(seed)
+    w = (torch.randn(G, N, K, generator=g) * 0.02).to(torch.bfloat16)
+    qs = [orc.quant_weight_128x128(w[i]) for i in range(G)]
+    return torch.stack([q for q, _ in qs]), torch.stack([s for _, s in qs])
+
+
+@pytest.mark.parametrize('col_major_scales', [False, True])
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+def test_grouped_contiguous(dev, col_major_scales, out_dtype):
+    print(f'case contiguous col_major={col_major_scales} {out_dtype}', flush=True)
+    from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_contiguous
+    G, N, K = 4, 384, 512
+    counts = [128, 0, 384, 256]  # padded per-expert spans, one expert empty
+    M_sum = sum(counts)
+    g = helpers.gen(9)
+    a = torch.randn(M_sum, K, generator=g).to(torch.bfloat16)
+    a_q, a_s = orc.quant_act_1x128(a)
+    w_q, w_s = _make_grouped_weights(G, N, K, 10)
+    m_indices = torch.cat([torch.full((c, ), e, dtype=torch.int32) for e, c in enumerate(counts)])
+    m_indices[128:256] = -1  # one skipped block
+    sentinel = 777.0
+    ref = orc.grouped_contiguous_ref(a_q, a_s, w_q, w_s, torch.full((M_sum, N), sentinel), m_indices)
+
+    a_s_dev = a_s.to(dev)
+    if col_major_scales:  # the layout dlblas/kernels/quant_dequant.py:65-83 hands over
+        pad = -(-M_sum // 4) * 4
+        buf = torch.zeros(K // 128, pad, device=dev)
+        buf[:, :M_sum] = a_s_dev.t()
+        a_s_dev = buf.t()[:M_sum]
+        assert not a_s_dev.is_contiguous()
+    out = torch.full((M_sum, N), sentinel, dtype=out_dtype, device=dev)
+    m_grouped_fp8_gemm_nt_contiguous([a_q.to(dev), a_s_dev], (w_q.to(dev), w_s.to(dev)), out, m_indices.to(dev))
+    torch.cuda.synchronize()
+    assert torch.all(out[128:256] == sentinel), 'skipped block was written'
+    helpers.tolerance_check(out, ref, 'grouped contiguous')
+
+
+def test_grouped_masked(dev):
+    print('case masked', flush=True)
+    from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
+    G, M_max, N, K = 6, 256, 512, 384
+    g = helpers.gen(12)
+    masked_m = torch.tensor([0, 1, 256, 130, 77, 128], dtype=torch.int32)
+    a = torch.randn(G, M_max, K, generator=g).to(torch.bfloat16)
+    a_q, a_s = orc.quant_act_1x128(a)
+    w_q, w_s = _make_grouped_weights(G, N, K, 13)
+    # rows at or beyond masked_m hold NaN codes and NaN scales: they must never reach a valid output
+    a_bits = a_q.view(torch.uint8).clone()
+    for e in range(G):
+        a_bits[e, int(masked_m[e]):] = 0x7F
+        a_s[e, int(masked_m[e]):] = float('nan')
+    a_q = a_bits.view(torch.float8_e4m3fn)
+    sentinel = -555.0
+    ref = orc.grouped_masked_ref(a_q, a_s, w_q, w_s, torch.full((G, M_max, N), sentinel), masked_m)
+    out = torch.full((G, M_max, N), sentinel, dtype=torch.bfloat16, device=dev)
+    m_grouped_fp8_gemm_nt_masked((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, masked_m.to(dev), 128)
+    torch.cuda.synchronize()
+    for e in range(G):
+        assert torch.all(out[e, int(masked_m[e]):] == sentinel), f'expert {e}: rows beyond masked_m were written'
+    assert not torch.isnan(out.float()).any()
+    helpers.tolerance_check(out, ref, 'grouped masked')
+
+
+def test_registry_selects_and_caches_on_gpu(dev):
+    print('case registry', flush=True)
+    from dlblas_amd import get_op
+    a_q, a_s, b_q, b_s = (t.to(dev) for t in helpers.make_dense(64, 512, 1024))
+    op = get_op('fp8_gemm', (a_q, b_q, a_s, b_s))
+    assert get_op('fp8_gemm', (a_q, b_q, a_s, b_s)) is op
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        out = op(a_q, b_q, a_s, b_s)
+    finally:
+        torch.set_default_dtype(prev)
+    ref = orc.dequant_ref(a_q.cpu(), a_s.cpu(), b_q.cpu(), b_s.cpu())
+    helpers.tolerance_check(out, ref, 'registry')
