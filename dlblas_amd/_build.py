@@ -12,7 +12,7 @@ SOURCES = ['dlblas_fp8_gemm.hip']
 # packed fp32 VALU forms are switched off for every device compile of this library
 HIPCC_FLAGS = [
     '-O3', '-std=c++17', '--offload-arch=gfx950', '-shared', '-fPIC', '-Xclang', '-target-feature', '-Xclang',
-    '-packed-fp32-ops', '-Wall', '-Wno-unused-function'
+    '-packed-fp32-ops', '-mllvm', '-amdgpu-mfma-vgpr-form=1', '-Wall', '-Wno-unused-function'
 ]
 
 

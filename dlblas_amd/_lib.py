@@ -33,6 +33,7 @@ SYMBOLS = {
     'dlb_fp8_gemm_grouped_masked':
     (ctypes.c_int, [_c_vp] * 6 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 3 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
+    'dlb_fp8_gemm_force_splitk': (ctypes.c_int, [ctypes.c_int]),
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
 }
 
@@ -116,6 +117,11 @@ def force_variant(name_or_id) -> None:
     if isinstance(name_or_id, str):
         name_or_id = variant_names().index(name_or_id)
     check(lib.dlb_fp8_gemm_force_variant(int(name_or_id)))
+
+
+def force_splitk(splitk) -> None:
+    """Pin the number of K splits of later dense calls from this thread (None or 0: heuristic)."""
+    check(load().dlb_fp8_gemm_force_splitk(int(splitk or 0)))
 
 
 def out_code(dtype: torch.dtype) -> int:

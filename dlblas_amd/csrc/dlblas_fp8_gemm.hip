@@ -8,6 +8,7 @@
 #include <cstring>
 
 #include "fp8_gemm_common.h"
+#include "fp8_gemm_pipelined.h"
 #include "fp8_gemm_skinny.h"
 #include "fp8_gemm_tiled.h"
 
@@ -46,6 +47,7 @@ namespace {
 
 thread_local char g_err[256] = "";
 thread_local int g_forced_variant = -1;
+thread_local int g_forced_splitk = 0;
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -62,11 +64,15 @@ enum Variant : int {
   kVarTile128x64,
   kVarSkinny16,
   kVarSkinny32,
+  kVarPipe256x128,
+  kVarPipe128x256,
+  kVarPipe256x256,
+  kVarPipe128x256w8,
   kVarCount
 };
 
 const char* const kVariantNames[kVarCount] = {
-    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32",
+    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8",
 };
 
 typedef TileCfg<128, 128, 2, 2> Tile128x128;
@@ -74,6 +80,10 @@ typedef TileCfg<64, 128, 2, 2> Tile64x128;
 typedef TileCfg<128, 64, 2, 2> Tile128x64;
 typedef SkinnyCfg<1, 4> Skinny16;
 typedef SkinnyCfg<2, 4> Skinny32;
+typedef PipeCfg<2, 2, 4, 2, 3> Pipe256x128;
+typedef PipeCfg<2, 2, 2, 4, 3> Pipe128x256;
+typedef PipeCfg<4, 2, 2, 4, 2> Pipe256x256;    // 8 waves, wave tile 64 x 128
+typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
 
 constexpr int kMaxDevices = 64;
 
@@ -125,6 +135,28 @@ hipError_t launch_tiled_mode(int mode, const Args& args, int grid, int dev, hipS
   }
 }
 
+template <class Cfg, int MODE>
+hipError_t launch_pipelined(const Args& args, int grid, int dev, hipStream_t stream) {
+  static std::atomic<unsigned long long> lds_done{0};
+  auto kernel = fp8_gemm_pipelined_kernel<Cfg, MODE>;
+  hipError_t e = ensure_lds(kernel, Cfg::LDS_BYTES, dev, &lds_done);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+  return hipGetLastError();
+}
+
+template <class Cfg>
+hipError_t launch_pipelined_mode(int mode, const Args& args, int grid, int dev, hipStream_t stream) {
+  switch (mode) {
+    case kDense:
+      return launch_pipelined<Cfg, kDense>(args, grid, dev, stream);
+    case kContiguous:
+      return launch_pipelined<Cfg, kContiguous>(args, grid, dev, stream);
+    default:
+      return launch_pipelined<Cfg, kMasked>(args, grid, dev, stream);
+  }
+}
+
 template <class Cfg>
 hipError_t launch_skinny(const Args& args, hipStream_t stream) {
   hipLaunchKernelGGL(fp8_gemm_skinny_kernel<Cfg>, dim3(args.tiles_n * args.splitk), dim3(Cfg::NT), 0, stream, args);
@@ -153,12 +185,23 @@ void tile_dims(int variant, int* bm, int* bn) {
     case kVarSkinny32:
       *bm = 32, *bn = 16;
       break;
+    case kVarPipe256x128:
+      *bm = 256, *bn = 128;
+      break;
+    case kVarPipe128x256:
+    case kVarPipe128x256w8:
+      *bm = 128, *bn = 256;
+      break;
+    case kVarPipe256x256:
+      *bm = 256, *bn = 256;
+      break;
     default:
       *bm = 128, *bn = 128;
   }
 }
 
 bool is_skinny(int v) { return v == kVarSkinny16 || v == kVarSkinny32; }
+bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe128x256w8; }
 
 // Largest split count (<= limit) whose slices still hold `min_kb` K blocks each.
 int pick_splitk(int64_t units, int kblocks, int cus, int waves_per_unit, int min_kb, int limit) {
@@ -188,11 +231,14 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
       v = kVarTile128x128;
   }
   if (K % 16 != 0) v = kVarExact;
+  if (is_pipelined(v) && (K % kScaleBlock != 0 || K == 0)) v = kVarTile128x128;  // DMA path moves whole K blocks
+  if (v == kVarPipe256x128 && mode == kContiguous) v = kVarPipe128x256;       // a tile must not straddle experts
+  if (v == kVarPipe256x256 && mode == kContiguous) v = kVarPipe128x256w8;
   if (is_skinny(v) && (mode != kDense || M > (v == kVarSkinny16 ? 16 : 32))) v = kVarTile128x128;
   if (v == kVarExact && mode != kDense) v = kVarTile128x128;
   pl.variant = v;
   tile_dims(v, &pl.bm, &pl.bn);
-  if (mode != kDense || v == kVarExact || kblocks < 2) return pl;
+  if (mode != kDense || v == kVarExact || kblocks < 2 || is_pipelined(v)) return pl;
 
   const int64_t tiles_n = ceil_div(N, pl.bn);
   const size_t avail = ws_bytes > DLB_WS_COUNTER_BYTES ? ws_bytes - DLB_WS_COUNTER_BYTES : 0;
@@ -271,6 +317,7 @@ int run(const Problem& pr) {
   if (cus < 0) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
 
   Plan pl = make_plan(pr.mode, pr.rows, pr.N, pr.K, cus, pr.ws ? pr.ws_bytes : 0);
+  if (g_forced_splitk > 0 && pr.mode == kDense && pl.variant != kVarExact) pl.splitk = g_forced_splitk;
   if (pl.splitk > 1) {
     if (!pr.ws || pr.ws_bytes < DLB_WS_COUNTER_BYTES) pl.splitk = 1;
     if (misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
@@ -336,7 +383,15 @@ int run(const Problem& pr) {
       }
       if (grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)grid);
       const int g = static_cast<int>(grid);
-      if (pl.variant == kVarTile64x128)
+      if (pl.variant == kVarPipe256x128)
+        e = launch_pipelined_mode<Pipe256x128>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarPipe128x256)
+        e = launch_pipelined_mode<Pipe128x256>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarPipe256x256)
+        e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarPipe128x256w8)
+        e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarTile64x128)
         e = launch_tiled_mode<Tile64x128>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarTile128x64)
         e = launch_tiled_mode<Tile128x64>(pr.mode, ar, g, dev, pr.stream);
@@ -363,11 +418,13 @@ const char* dlb_last_error(void) { return dlb::g_err; }
 size_t dlb_fp8_gemm_workspace_bytes(int64_t rows, int64_t N, int64_t K) {
   (void)K;
   if (rows <= 0 || N <= 0) return DLB_WS_COUNTER_BYTES;
-  // Split-K is only used while the un-split grid cannot fill the chip, i.e. for at most ~256 tiles of
-  // 128 x 128 fp32 partials times at most 16 splits; small-M problems need far less.
-  const int64_t tiles = dlb::ceil_div(rows, 64) * dlb::ceil_div(N, 64);
-  const int64_t capped = tiles < 1024 ? tiles : 1024;
-  return DLB_WS_COUNTER_BYTES + static_cast<size_t>(capped) * 64 * 64 * sizeof(float) * 16;
+  // Split-K only runs while the un-split grid cannot fill the chip, so (tiles x splits) stays within a few
+  // hundred fp32 tiles of at most 128 x 128: 32 MiB covers every plan; the planner lowers the split count to
+  // fit whatever it is given.
+  const size_t cap = static_cast<size_t>(32) << 20;
+  const int64_t padded = dlb::ceil_div(rows, 128) * dlb::ceil_div(N, 128);
+  const size_t want = padded > 1024 ? cap : static_cast<size_t>(padded) * 128 * 128 * sizeof(float) * 16;
+  return DLB_WS_COUNTER_BYTES + (want < cap ? want : cap);
 }
 
 int dlb_fp8_gemm(const void* a, const void* b, const float* a_s, const float* b_s, void* c, int64_t M, int64_t N,
@@ -400,6 +457,12 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
 int dlb_fp8_gemm_force_variant(int variant) {
   if (variant >= dlb::kVarCount) return dlb::fail(DLB_ERR_BAD_SHAPE, "unknown kernel variant %d", variant);
   dlb::g_forced_variant = variant < 0 ? -1 : variant;
+  return DLB_OK;
+}
+
+int dlb_fp8_gemm_force_splitk(int splitk) {
+  if (splitk < 0 || splitk > 64) return dlb::fail(DLB_ERR_BAD_SHAPE, "split count %d outside [0, 64]", splitk);
+  dlb::g_forced_splitk = splitk;
   return DLB_OK;
 }
 

@@ -1,0 +1,333 @@
+// Compute-bound FP8 block-scaled GEMM for gfx950: 32x32x64 e4m3 MFMA, tiles streamed HBM -> LDS by the DMA
+// path of the memory pipeline (global_load_lds_dwordx4, no VGPR staging), multi-stage LDS ring, one barrier
+// per 128-wide K step, block scales applied with one FMA per accumulator element and K step.
+//
+// Workgroup = WGM x WGN waves, one wave per SIMD; a wave owns MF x NF fragments of 32 x 32 outputs.
+// MFMA operand roles: "A" = 32 rows of the weight tile (n), "B" = 32 rows of the activation tile (m), so a lane's
+// 16 accumulator components of a fragment are 4 groups of 4 consecutive n for ONE m (= lane & 31): the activation
+// scale is one value per lane and fragment row block, and every lane stores 4 contiguous outputs at a time.
+//
+// Arithmetic: fp8_gemm_kernel of the reference (dlblas/kernels/fp8_gemm.py:49-60).  Requires K % 128 == 0.
+#pragma once
+
+#include "fp8_gemm_common.h"
+#include "fp8_gemm_tiled.h"  // xcd_remap
+
+namespace dlb {
+
+// D = A_op * B_op^T, A_op / B_op [32 x 64] e4m3: lane l supplies row (l & 31), 32 K-bytes selected by (l >> 5).
+// Lane l receives D[8 * (t / 4) + 4 * (l >> 5) + (t % 4)][l & 31] in component t.
+__device__ __forceinline__ v16f mfma_32x32x64_e4m3(v8i a_op, v8i b_op, v16f c) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_op, b_op, c, 0, 0, 0, 0, 0, 0);
+}
+
+// XOR pattern of the 16-byte chunk index inside a 128-byte LDS row: distinct within any 8 consecutive rows, and
+// rows r and r + 8 that share a pattern differ in row parity, i.e. in the 128-byte half of a 256-byte bank line.
+__device__ __forceinline__ int chunk_swizzle(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+__device__ __forceinline__ int lds_off32(int row, int chunk) {
+  return row * kScaleBlock + ((chunk ^ chunk_swizzle(row)) << 4);
+}
+
+// A lane reads four 16-byte chunks of "its" row (lane & 31) of every 32-row fragment: logical chunks 2 h, 2 h + 1
+// (K half 0) and 4 + 2 h, 5 + 2 h (K half 1), h = lane >> 5.  Fragments start at multiples of 32 rows, which leaves
+// the swizzle untouched, so these four byte offsets are the same for every fragment of every tile.
+struct LaneChunks {
+  int off[4];
+};
+
+__device__ __forceinline__ LaneChunks make_lane_chunks(int l32, int h) {
+  LaneChunks lc;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) lc.off[i] = lds_off32(l32, (i >> 1) * 4 + 2 * h + (i & 1));
+  return lc;
+}
+
+// 8 VGPRs = the 32 operand bytes of one lane for the fragment whose first row starts `frag_bytes` into the LDS
+// ring (wave-uniform) and K half `kk` of the 128-byte step.
+__device__ __forceinline__ v8i lds_read_frag32(const uint8_t* ring, int frag_bytes, const LaneChunks& lc, int kk) {
+  const v4i lo = *reinterpret_cast<const v4i*>(ring + frag_bytes + lc.off[2 * kk]);
+  const v4i hi = *reinterpret_cast<const v4i*>(ring + frag_bytes + lc.off[2 * kk + 1]);
+  return v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+
+// One wave-wide DMA: lane i moves 16 bytes from (base + voff) to lds_dst + 16 i.
+__device__ __forceinline__ void dma_16(const uint8_t* base, uint32_t voff, uint8_t* lds_dst) {
+  __builtin_amdgcn_global_load_lds((global_ptr_t)(base + voff), (lds_ptr_t)lds_dst, 16, 0, 0);
+}
+// lane i moves 4 bytes from (base + voff) to lds_dst + 4 i.
+__device__ __forceinline__ void dma_4(const uint8_t* base, uint32_t voff, uint8_t* lds_dst) {
+  __builtin_amdgcn_global_load_lds((global_ptr_t)(base + voff), (lds_ptr_t)lds_dst, 4, 0, 0);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // s_waitcnt with only vmcnt constrained: vmcnt = simm16[3:0] | simm16[15:14] << 4, expcnt [6:4], lgkmcnt [11:8]
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | (((N >> 4) & 0x3) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// Workgroup barrier that orders LDS traffic only: every wave's LDS reads have returned (lgkmcnt) before it
+// arrives.  Unlike __syncthreads() it does not drain the vector-memory counter, so DMA groups that were issued
+// for later stages stay in flight across it; the caller waits for the group it needs with wait_vmcnt first.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_>
+struct PipeCfg {
+  static constexpr int WGM = WGM_, WGN = WGN_, MF = MF_, NF = NF_, STAGES = STAGES_;
+  static constexpr int WAVES = WGM * WGN;
+  static constexpr int NT = WAVES * 64;
+  static constexpr int BM = WGM * MF * 32;
+  static constexpr int BN = WGN * NF * 32;
+  static constexpr int A_INST = BM / 8 / WAVES;  // 16-byte DMA instructions per wave and stage for the A tile
+  static constexpr int B_INST = BN / 8 / WAVES;
+  static constexpr int S_INST = (BM + NT - 1) / NT;  // 4-byte DMA instructions per wave for the a_s slice
+  static constexpr int A_BYTES = BM * kScaleBlock;
+  static constexpr int B_BYTES = BN * kScaleBlock;
+  static constexpr int S_BYTES = S_INST * NT * 4;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + S_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int LOADS_PER_STAGE = A_INST + B_INST + S_INST;  // vmcnt units per wave and stage
+  static_assert(BM % (8 * WAVES) == 0 && BN % (8 * WAVES) == 0, "tile rows must divide over the DMA instructions");
+  static_assert(NF * 32 <= 128 && 128 % (NF * 32) == 0, "a wave's n span must stay inside one 128-wide scale block");
+  static_assert(LOADS_PER_STAGE * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+};
+
+template <class Cfg, int MODE>
+__global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args p) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, MF = Cfg::MF, NF = Cfg::NF, WAVES = Cfg::WAVES, STAGES = Cfg::STAGES;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int h = lane >> 5;
+  const int wm0 = (wave / Cfg::WGN) * (MF * 32);
+  const int wn0 = (wave % Cfg::WGN) * (NF * 32);
+  const LaneChunks lc = make_lane_chunks(l32, h);
+
+  const int tiles = p.tiles_m * p.tiles_n;
+  int walk_g = 0;
+  int walk_base = 0;
+
+  for (int vb = blockIdx.x;; vb += gridDim.x) {
+    int g = 0, mt, nt, m_end;
+    if (MODE == kMasked) {
+      int mtiles = 0;
+      while (walk_g < p.G) {
+        const int valid = min(max(p.gidx[walk_g], 0), p.M);
+        mtiles = (valid + BM - 1) / BM;
+        const int cnt = mtiles * p.tiles_n;
+        if (vb < walk_base + cnt) break;
+        walk_base += cnt;
+        ++walk_g;
+      }
+      if (walk_g >= p.G) break;
+      g = walk_g;
+      const int local = vb - walk_base;
+      mt = local % mtiles;
+      nt = local / mtiles;
+      m_end = min(max(p.gidx[g], 0), p.M);
+    } else {
+      if (vb >= tiles) break;
+      const int t = xcd_remap(vb, tiles);
+      const int width = p.group_m * p.tiles_n;
+      const int grp = t / width;
+      const int first_m = grp * p.group_m;
+      const int gsz = min(p.tiles_m - first_m, p.group_m);
+      const int in_grp = t - grp * width;
+      mt = first_m + in_grp % gsz;
+      nt = in_grp / gsz;
+      m_end = p.M;
+      if (MODE == kContiguous) {
+        g = p.gidx[mt * BM];
+        if (g < 0 || g >= p.G) continue;
+      }
+    }
+    g = __builtin_amdgcn_readfirstlane(g);
+    const int m0 = __builtin_amdgcn_readfirstlane(mt * BM);
+    const int n0 = __builtin_amdgcn_readfirstlane(nt * BN);
+
+    const int64_t esz = p.out_f32 ? 4 : 2;
+    const uint8_t* a_tile = p.a + static_cast<int64_t>(m0) * p.K;
+    const float* as_tile = p.a_s + static_cast<int64_t>(m0) * p.as_sm;
+    char* c_base = static_cast<char*>(p.c);
+    if (MODE == kMasked) {
+      a_tile += static_cast<int64_t>(g) * p.a_gs;
+      as_tile += static_cast<int64_t>(g) * p.as_gs;
+      c_base += static_cast<int64_t>(g) * p.c_gs * esz;
+    }
+    const uint8_t* b_tile = p.b + static_cast<int64_t>(g) * p.b_gs + static_cast<int64_t>(n0) * p.K;
+    const int nblk = __builtin_amdgcn_readfirstlane(min((n0 + wn0) / kScaleBlock, p.nblocks - 1));
+    const float* bs_row = p.b_s + static_cast<int64_t>(g) * p.bs_gs + static_cast<int64_t>(nblk) * p.kblocks;
+
+    // DMA addressing.  Instruction j of this wave fills LDS rows 8 (j WAVES + wave) .. + 7; lane i fills physical
+    // chunk (i & 7) of row (i >> 3), which holds logical chunk (i & 7) ^ swizzle(row).  WAVES is even, so the
+    // swizzle does not depend on j and one per-lane chunk offset serves every instruction; the row part is
+    // recomputed per instruction (two VALU ops) instead of being kept in registers.  Rows past the valid range
+    // re-read the last valid row.
+    static_assert(WAVES % 2 == 0, "chunk swizzle must not depend on the DMA instruction index");
+    const int a_last = m_end - 1 - m0;
+    const int b_last = p.N - 1 - n0;
+    const int dma_row = 8 * wave + (lane >> 3);
+    const uint32_t dma_chunk = static_cast<uint32_t>(((lane & 7) ^ chunk_swizzle(dma_row)) * 16);
+    const uint32_t uK = static_cast<uint32_t>(p.K);
+
+    auto issue_stage = [&](int kb, int stage) {
+      uint8_t* sbase = smem + stage * Cfg::STAGE_BYTES;
+      const uint8_t* ag = a_tile + static_cast<int64_t>(kb) * kScaleBlock;
+      const uint8_t* bg = b_tile + static_cast<int64_t>(kb) * kScaleBlock;
+      const uint8_t* sg = reinterpret_cast<const uint8_t*>(as_tile + static_cast<int64_t>(kb) * p.as_sk);
+#pragma unroll
+      for (int j = 0; j < Cfg::A_INST; ++j) {
+        const uint32_t off = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, a_last)) * uK + dma_chunk;
+        dma_16(ag, off, sbase + (j * WAVES + wave) * 1024);
+      }
+#pragma unroll
+      for (int j = 0; j < Cfg::B_INST; ++j) {
+        const uint32_t off = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, b_last)) * uK + dma_chunk;
+        dma_16(bg, off, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
+      }
+#pragma unroll
+      for (int j = 0; j < Cfg::S_INST; ++j) {
+        const int row = (j * WAVES + wave) * 64 + lane;
+        const uint32_t off = static_cast<uint32_t>(min(row, a_last)) * static_cast<uint32_t>(p.as_sm) * 4u;
+        dma_4(sg, off, sbase + Cfg::A_BYTES + Cfg::B_BYTES + (j * WAVES + wave) * 256);
+      }
+    };
+
+    v16f acc[MF][NF];
+#pragma unroll
+    for (int mi = 0; mi < MF; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < NF; ++ni)
+#pragma unroll
+        for (int t = 0; t < 16; ++t) acc[mi][ni][t] = 0.f;
+
+    const int nk = p.kblocks;
+    __syncthreads();  // the previous tile's readers are done with the ring
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+      if (s < nk) issue_stage(s, s);
+
+    // weight scales of this wave's n block: 64 K blocks per refill, one per lane, picked out with v_readlane
+    float bs_cache = 0.f;
+    constexpr int T = MF * NF;
+    int stage = 0;
+    for (int kb = 0; kb < nk; ++kb) {
+      if ((kb & 63) == 0) {
+        // refill the scale cache; the explicit drain keeps the compiler from waiting on this load (and with it
+        // on every DMA group in flight) at each later use
+        bs_cache = bs_row[min(kb + lane, nk - 1)];
+        wait_vmcnt<0>();
+        asm volatile("" : "+v"(bs_cache));
+      }
+      // stage kb's DMA is the oldest group in flight; at most STAGES - 2 younger groups may stay outstanding
+      const int younger = min(nk - 1 - kb, STAGES - 2);
+      if (younger >= 2)
+        wait_vmcnt<2 * Cfg::LOADS_PER_STAGE>();
+      else if (younger == 1)
+        wait_vmcnt<Cfg::LOADS_PER_STAGE>();
+      else
+        wait_vmcnt<0>();
+      lds_barrier();
+      if (kb + STAGES - 1 < nk) {
+        int fill = stage + STAGES - 1;
+        if (fill >= STAGES) fill -= STAGES;
+        issue_stage(kb + STAGES - 1, fill);
+      }
+
+      const int a_frag0 = stage * Cfg::STAGE_BYTES + wm0 * kScaleBlock;                 // wave-uniform byte offsets
+      const int b_frag0 = stage * Cfg::STAGE_BYTES + Cfg::A_BYTES + wn0 * kScaleBlock;
+      const float* sS = reinterpret_cast<const float*>(smem + stage * Cfg::STAGE_BYTES + Cfg::A_BYTES + Cfg::B_BYTES);
+      const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bs_cache), kb & 63));
+      constexpr int kFragBytes = 32 * kScaleBlock;
+
+      float sc[MF];
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) sc[mi] = sS[wm0 + mi * 32 + l32] * sb;
+
+      // The scale FMAs of a fragment are issued after the MFMAs of the next one so that they run under them.
+      v16f part[2];
+      if (MF >= NF) {
+        // keep the wave's weight fragments in registers, stream the activation fragments past them
+        v8i wf[NF][2];
+        v8i xf[2];
+#pragma unroll
+        for (int ni = 0; ni < NF; ++ni) {
+          wf[ni][0] = lds_read_frag32(smem, b_frag0 + ni * kFragBytes, lc, 0);
+          wf[ni][1] = lds_read_frag32(smem, b_frag0 + ni * kFragBytes, lc, 1);
+        }
+        xf[0] = lds_read_frag32(smem, a_frag0, lc, 0);
+        xf[1] = lds_read_frag32(smem, a_frag0, lc, 1);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          const int mi = t / NF, ni = t % NF;
+          v16f z;
+#pragma unroll
+          for (int u = 0; u < 16; ++u) z[u] = 0.f;
+          z = mfma_32x32x64_e4m3(wf[ni][0], xf[0], z);
+          part[t & 1] = mfma_32x32x64_e4m3(wf[ni][1], xf[1], z);
+          if (ni == NF - 1 && mi + 1 < MF) {  // last use of this activation fragment has been issued: reload in place
+            xf[0] = lds_read_frag32(smem, a_frag0 + (mi + 1) * kFragBytes, lc, 0);
+            xf[1] = lds_read_frag32(smem, a_frag0 + (mi + 1) * kFragBytes, lc, 1);
+          }
+          if (t > 0) acc[(t - 1) / NF][(t - 1) % NF] += part[(t - 1) & 1] * sc[(t - 1) / NF];
+        }
+        acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc[MF - 1];
+      } else {
+        // fewer activation fragments than weight fragments: keep the activations, stream the weights
+        v8i xf[MF][2];
+        v8i wf[2];
+#pragma unroll
+        for (int mi = 0; mi < MF; ++mi) {
+          xf[mi][0] = lds_read_frag32(smem, a_frag0 + mi * kFragBytes, lc, 0);
+          xf[mi][1] = lds_read_frag32(smem, a_frag0 + mi * kFragBytes, lc, 1);
+        }
+        wf[0] = lds_read_frag32(smem, b_frag0, lc, 0);
+        wf[1] = lds_read_frag32(smem, b_frag0, lc, 1);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+          const int ni = t / MF, mi = t % MF;
+          v16f z;
+#pragma unroll
+          for (int u = 0; u < 16; ++u) z[u] = 0.f;
+          z = mfma_32x32x64_e4m3(wf[0], xf[mi][0], z);
+          part[t & 1] = mfma_32x32x64_e4m3(wf[1], xf[mi][1], z);
+          if (mi == MF - 1 && ni + 1 < NF) {  // last use of this weight fragment has been issued: reload in place
+            wf[0] = lds_read_frag32(smem, b_frag0 + (ni + 1) * kFragBytes, lc, 0);
+            wf[1] = lds_read_frag32(smem, b_frag0 + (ni + 1) * kFragBytes, lc, 1);
+          }
+          if (t > 0) acc[(t - 1) % MF][(t - 1) / MF] += part[(t - 1) & 1] * sc[(t - 1) % MF];
+        }
+        acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc[MF - 1];
+      }
+      stage = stage + 1 == STAGES ? 0 : stage + 1;
+    }
+
+    // epilogue: lane holds c[m0 + wm0 + 32 mi + (lane & 31)][n0 + wn0 + 32 ni + 8 u + 4 (lane >> 5) + 0..3], u = 0..3
+#pragma unroll
+    for (int mi = 0; mi < MF; ++mi) {
+      const int m = m0 + wm0 + mi * 32 + l32;
+      if (m >= m_end) continue;
+      char* c_row = c_base + static_cast<int64_t>(m) * p.N * esz;
+#pragma unroll
+      for (int ni = 0; ni < NF; ++ni) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int n = n0 + wn0 + ni * 32 + u * 8 + h * 4;
+          const v4f v = {acc[mi][ni][4 * u], acc[mi][ni][4 * u + 1], acc[mi][ni][4 * u + 2], acc[mi][ni][4 * u + 3]};
+          if (p.out_f32)
+            store_row4<true>(c_row, n, v, p.N - n, p.vec_store);
+          else
+            store_row4<false>(c_row, n, v, p.N - n, p.vec_store);
+        }
+      }
+    }
+  }
+}
+
+}  // namespace dlb

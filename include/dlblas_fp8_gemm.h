@@ -148,6 +148,12 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
  */
 int dlb_fp8_gemm_force_variant(int variant);
 
+/*
+ * Tuning / test hook: force the number of K splits of the next dense calls FROM THIS THREAD (clamped to what the
+ * workspace and K allow); 0 restores the heuristic.  Grouped calls never split K.
+ */
+int dlb_fp8_gemm_force_splitk(int splitk);
+
 /* Name of kernel variant `variant`, or NULL beyond the last one. */
 const char* dlb_fp8_gemm_variant_name(int variant);
 

@@ -61,7 +61,8 @@ def e4m3fn_table() -> np.ndarray:
     out = np.empty(256, dtype=np.float32)
     for code in range(256):
         try:
-            out[code] = np.float32(float(e4m3fn_value(code)))
+            value = float(e4m3fn_value(code))
+            out[code] = np.float32(-0.0 if (code == 0x80) else value)  # a Fraction cannot carry the sign of zero
         except ValueError:
             out[code] = np.float32('nan')
     return out

@@ -1,0 +1,256 @@
+"""Pins the CPU oracle (oracle/fp8_block_gemm.py, oracle/fp8_gemm_oracle.c) without a GPU.
+
+Every check is chosen so that a plausible mistake in the oracle (wrong bias, dropped scale, transposed operand,
+wrong block index, missing clamp) fails it.
+"""
+import ctypes
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+from oracle import fp8_block_gemm as orc
+from oracle.build_oracle import LIB_PATH, build_oracle
+
+
+@pytest.fixture(scope='module')
+def c_oracle():
+    import os
+    if not os.path.exists(LIB_PATH):
+        build_oracle()
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.dlb_oracle_e4m3fn_to_f32.restype = ctypes.c_float
+    lib.dlb_oracle_e4m3fn_to_f32.argtypes = [ctypes.c_uint8]
+    lib.dlb_oracle_f32_to_bf16.restype = ctypes.c_uint16
+    lib.dlb_oracle_f32_to_bf16.argtypes = [ctypes.c_float]
+    lib.dlb_oracle_fp8_gemm.restype = None
+    lib.dlb_oracle_fp8_gemm.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int64] * 3
+    return lib
+
+
+def _c_gemm(lib, a_q, a_s, b_q, b_s):
+    M, K = a_q.shape
+    N = b_q.shape[0]
+    a = a_q.view(torch.uint8).contiguous()
+    b = b_q.view(torch.uint8).contiguous()
+    a_s, b_s = a_s.contiguous().float(), b_s.contiguous().float()
+    c = torch.empty(M, N, dtype=torch.float32)
+    lib.dlb_oracle_fp8_gemm(a.data_ptr(), b.data_ptr(), a_s.data_ptr(), b_s.data_ptr(), c.data_ptr(), M, N, K)
+    return c
+
+
+# ---------------------------------------------------------------- e4m3fn decode
+def test_decode_table_exhaustive_against_torch_and_definition(c_oracle):
+    codes = torch.arange(256, dtype=torch.uint8)
+    table = orc.decode_e4m3fn(codes)
+    via_torch = codes.view(torch.float8_e4m3fn).float()
+    for code in range(256):
+        c_val = c_oracle.dlb_oracle_e4m3fn_to_f32(code)
+        if code & 0x7F == 0x7F:
+            assert np.isnan(float(table[code])) and np.isnan(float(via_torch[code])) and np.isnan(c_val)
+            continue
+        exact = orc.e4m3fn_value(code)
+        assert Fraction(float(table[code])) == exact
+        assert float(via_torch[code]) == float(table[code]) == c_val
+    # landmarks of the format: max 448, min normal 2^-6, min subnormal 2^-9, signed zero
+    assert float(table[0x7E]) == 448.0 and float(table[0xFE]) == -448.0
+    assert float(table[0x08]) == 2.0**-6 and float(table[0x01]) == 2.0**-9
+    assert float(table[0x38]) == 1.0
+    assert float(table[0x00]) == 0.0 and float(table[0x80]) == 0.0 and np.signbit(table[0x80].item()) and np.signbit(via_torch[0x80].item())
+
+
+def test_bf16_rounding_restated_in_c(c_oracle):
+    g = helpers.gen(1)
+    x = torch.cat([torch.randn(4096, generator=g) * 10, torch.tensor([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3e38])])
+    want = x.to(torch.bfloat16).view(torch.int16).numpy().astype(np.uint16)
+    got = np.array([c_oracle.dlb_oracle_f32_to_bf16(float(v)) for v in x], dtype=np.uint16)
+    assert np.array_equal(want, got)
+
+
+# ---------------------------------------------------------------- dense GEMM
+@pytest.mark.parametrize('M,N,K', [(64, 512, 1024), (5, 200, 400), (1, 130, 128), (33, 129, 520)])
+def test_closed_form_equals_block_loop_and_c(c_oracle, M, N, K):
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K)
+    closed = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    looped = orc.dequant_ref_blocked(a_q, a_s, b_q, b_s)
+    in_c = _c_gemm(c_oracle, a_q, a_s, b_q, b_s)
+    scale = closed.abs().max()
+    assert (closed - looped).abs().max() <= 2e-6 * scale
+    assert (closed - in_c).abs().max() <= 2e-6 * scale
+
+
+def test_signed_scales_as_in_reference_test(c_oracle):
+    a_q, a_s, b_q, b_s = helpers.make_raw(64, 256, 512)
+    assert (a_s < 0).any() and (b_s < 0).any()
+    closed = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    in_c = _c_gemm(c_oracle, a_q, a_s, b_q, b_s)
+    assert (closed - in_c).abs().max() <= 1e-5 * closed.abs().max()
+
+
+def test_integer_inputs_are_exact():
+    g = helpers.gen(2)
+    M, N, K = 7, 140, 300
+    a = torch.randint(-6, 7, (M, K), generator=g)
+    b = torch.randint(-6, 7, (N, K), generator=g)
+    a_s = torch.randint(1, 4, (M, 3), generator=g).float()
+    b_s = torch.randint(1, 4, (2, 3), generator=g).float()
+    want = torch.zeros(M, N, dtype=torch.int64)
+    for m in range(M):
+        for n in range(N):
+            for kb in range(3):
+                ks = slice(kb * 128, min(K, (kb + 1) * 128))
+                want[m, n] += int((a[m, ks] * b[n, ks]).sum()) * int(a_s[m, kb]) * int(b_s[n // 128, kb])
+    got = orc.dequant_ref(a.float().to(torch.float8_e4m3fn), a_s, b.float().to(torch.float8_e4m3fn), b_s)
+    assert torch.equal(got.long(), want) and torch.equal(got, want.float())
+
+
+def test_one_hot_rows_select_dequantised_weight_columns():
+    """A row with a single 1.0 at column k0 must return b[:, k0] * b_s[n // 128, k0 // 128] * a_s[m, k0 // 128]:
+    catches a transposed operand, a wrong scale block index and a dropped scale."""
+    g = helpers.gen(4)
+    N, K = 300, 384
+    b = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+    b_q, b_s = orc.quant_weight_128x128(b)
+    ks = [0, 127, 128, 200, 383]
+    a = torch.zeros(len(ks), K)
+    for r, k0 in enumerate(ks):
+        a[r, k0] = 1.0
+    a_s = torch.tensor([[2.0, 3.0, 5.0]]).repeat(len(ks), 1)
+    out = orc.dequant_ref(a.to(torch.float8_e4m3fn), a_s, b_q, b_s)
+    deq_b = orc.decode_e4m3fn(b_q)
+    for r, k0 in enumerate(ks):
+        for n in (0, 127, 128, 299):
+            want = deq_b[n, k0] * b_s[n // 128, k0 // 128] * a_s[r, k0 // 128]
+            assert out[r, n] == pytest.approx(float(want), rel=1e-6)
+
+
+def test_unit_scales_reduce_to_plain_matmul():
+    a_q, _, b_q, _ = helpers.make_raw(32, 64, 256, scale_kind='ones')
+    out = orc.dequant_ref(a_q, torch.ones(32, 2), b_q, torch.ones(1, 2))
+    want = a_q.float().double() @ b_q.float().double().t()
+    assert (out.double() - want).abs().max() <= 1e-5 * want.abs().max()
+
+
+def test_output_cast_and_leading_dims():
+    a_q, a_s, b_q, b_s = helpers.make_dense(12, 128, 256)
+    flat = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    shaped = orc.dequant_ref(a_q.reshape(3, 4, 256), a_s.reshape(3, 4, 2), b_q, b_s, torch.bfloat16)
+    assert shaped.shape == (3, 4, 128) and shaped.dtype == torch.bfloat16
+    assert torch.equal(shaped.reshape(12, 128), flat.to(torch.bfloat16))
+
+
+# ---------------------------------------------------------------- quantisers
+def test_act_quantiser_invariants():
+    g = helpers.gen(5)
+    x = torch.randn(37, 512, generator=g).to(torch.bfloat16)
+    x[3, 128:256] = 0  # an all-zero group takes the eps scale
+    q, s = orc.quant_act_1x128(x)
+    assert q.dtype == torch.float8_e4m3fn and s.shape == (37, 4) and s.dtype == torch.float32
+    qf = orc.decode_e4m3fn(q).reshape(37, 4, 128)
+    xf = x.float().reshape(37, 4, 128)
+    assert not torch.isnan(qf).any() and qf.abs().max() <= 448
+    amax = xf.abs().amax(-1)
+    assert torch.allclose(s, amax.clamp_min(1e-10) / 448, rtol=1e-6, atol=0)
+    assert s[3, 1] == pytest.approx(1e-10 / 448, rel=1e-5) and (qf[3, 1] == 0).all()
+    nonzero = amax > 0
+    assert torch.all(qf.abs().amax(-1)[nonzero] == 448), 'the largest element of a group must map to +-448'
+    # reconstruction: half an e4m3 ulp of the scaled value (3 mantissa bits -> 2^-4 relative), subnormal floor 2^-10
+    recon = qf * s[..., None]
+    bound = torch.maximum(xf.abs() * 2.0**-4, s[..., None] * 2.0**-10) * 1.0001
+    assert torch.all((recon - xf).abs() <= bound)
+
+
+def test_weight_quantiser_blocks_and_ragged_edges():
+    g = helpers.gen(6)
+    w = (torch.randn(300, 200, generator=g) * 0.02).to(torch.bfloat16)
+    q, s = orc.quant_weight_128x128(w)
+    assert q.shape == (300, 200) and s.shape == (3, 2)
+    for nb in range(3):
+        for kb in range(2):
+            blk = w[nb * 128:(nb + 1) * 128, kb * 128:(kb + 1) * 128].float()
+            assert s[nb, kb] == pytest.approx(float(blk.abs().max()) / 448, rel=1e-6)
+            qb = orc.decode_e4m3fn(q[nb * 128:(nb + 1) * 128, kb * 128:(kb + 1) * 128])
+            assert qb.abs().max() == 448
+    recon = orc.decode_e4m3fn(q) * s.repeat_interleave(128, 0).repeat_interleave(128, 1)[:300, :200]
+    assert (recon - w.float()).abs().max() <= w.float().abs().max() * 2.0**-4
+
+
+def test_cast_is_round_to_nearest_even_and_clamp_is_needed():
+    """The e4m3 cast used by the quantisers is RTNE (checked against a brute-force nearest-value search with
+    ties to the even mantissa) and does not saturate, which is why the quantisers clamp first."""
+    table = orc.e4m3fn_table()
+    finite = np.array([c for c in range(256) if c & 0x7F != 0x7F and c != 0x80])
+    vals = table[finite].astype(np.float64)
+    g = helpers.gen(8)
+    x = torch.cat([torch.randn(2000, generator=g) * 100, torch.tensor([17.0, 19.0, 21.0, 0.0009765625 * 1.5, 447.9, -448.0])])
+    x = x.clamp(-448, 448)
+    got = x.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    for xv, code in zip(x.double().numpy(), got):
+        d = np.abs(vals - xv)
+        best = d.min()
+        cands = finite[d == best]
+        if len(cands) > 1:
+            cands = [c for c in cands if c & 1 == 0]
+        assert table[code] == table[cands[0]], f'{xv}: cast gave {table[code]}, nearest-even is {table[cands[0]]}'
+    assert torch.isnan(torch.tensor([500.0]).to(torch.float8_e4m3fn).float()).all()
+
+
+# ---------------------------------------------------------------- grouped
+def test_grouped_contiguous_is_per_block_dense():
+    g = helpers.gen(14)
+    G, N, K = 3, 160, 256
+    w_q, w_s = zip(*[orc.quant_weight_128x128((torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16))
+                     for _ in range(G)])
+    w_q, w_s = torch.stack(w_q), torch.stack(w_s)
+    a_q, a_s = orc.quant_act_1x128(torch.randn(300, K, generator=g).to(torch.bfloat16))
+    m_indices = torch.tensor([2] * 128 + [-1] * 128 + [0] * 44, dtype=torch.int32)
+    out = orc.grouped_contiguous_ref(a_q, a_s, w_q, w_s, torch.full((300, N), 9.0), m_indices)
+    assert torch.equal(out[:128], orc.dequant_ref(a_q[:128], a_s[:128], w_q[2], w_s[2]))
+    assert torch.all(out[128:256] == 9.0)
+    assert torch.equal(out[256:], orc.dequant_ref(a_q[256:], a_s[256:], w_q[0], w_s[0]))
+
+
+def test_grouped_masked_ignores_rows_beyond_mask():
+    g = helpers.gen(15)
+    G, M_max, N, K = 3, 64, 128, 256
+    w_q, w_s = zip(*[orc.quant_weight_128x128((torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16))
+                     for _ in range(G)])
+    w_q, w_s = torch.stack(w_q), torch.stack(w_s)
+    a_q, a_s = orc.quant_act_1x128(torch.randn(G, M_max, K, generator=g).to(torch.bfloat16))
+    masked_m = torch.tensor([0, 64, 17], dtype=torch.int32)
+    bits = a_q.view(torch.uint8).clone()
+    bits[2, 17:] = 0x7F
+    out = orc.grouped_masked_ref(bits.view(torch.float8_e4m3fn), a_s, w_q, w_s, torch.full((G, M_max, N), -3.0), masked_m)
+    assert torch.all(out[0] == -3.0) and torch.all(out[2, 17:] == -3.0) and not torch.isnan(out).any()
+    assert torch.equal(out[1], orc.dequant_ref(a_q[1], a_s[1], w_q[1], w_s[1]))
+    assert torch.equal(out[2, :17], orc.dequant_ref(a_q[2, :17], a_s[2, :17], w_q[2], w_s[2]))
+
+
+# ---------------------------------------------------------------- metrics
+def test_error_metrics():
+    ref = torch.tensor([1.0, -2.0, 0.0, 4.0])
+    out = torch.tensor([1.01, -2.0, 0.0005, 4.0])
+    rms = float(ref.pow(2).mean().sqrt())
+    assert orc.max_rel_err(out, ref, 1e-3) == pytest.approx(max(0.01, 0.0005 / (1e-3 * rms)), rel=1e-5)
+    assert orc.similarity_gap(ref, ref) == 0.0
+    assert orc.similarity_gap(ref, -ref) == pytest.approx(2.0)
+
+
+def test_golden_fixture_matches_oracle():
+    """Committed seeded vectors (tests/golden/make_golden.py wrote them from this oracle): guards the oracle and
+    the input generators against silent drift between rounds and machines."""
+    import json
+    import os
+    path = os.path.join(os.path.dirname(__file__), 'golden', 'fp8_gemm_golden.json')
+    with open(path) as fh:
+        golden = json.load(fh)
+    for case in golden['cases']:
+        a_q, a_s, b_q, b_s = helpers.make_dense(case['M'], case['N'], case['K'], seed=case['seed'])
+        ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+        assert int(a_q.view(torch.uint8).long().sum()) == case['a_q_bytesum']
+        assert int(b_q.view(torch.uint8).long().sum()) == case['b_q_bytesum']
+        for (m, n, v) in case['samples']:
+            assert float(ref[m, n]) == pytest.approx(v, rel=1e-5, abs=1e-7)
+        assert float(ref.double().sum()) == pytest.approx(case['sum'], rel=1e-5, abs=1e-4)
