@@ -68,11 +68,12 @@ enum Variant : int {
   kVarPipe128x256,
   kVarPipe256x256,
   kVarPipe128x256w8,
+  kVarPipe256x256p2,
   kVarCount
 };
 
 const char* const kVariantNames[kVarCount] = {
-    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8",
+    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8", "pipe256x256p2",
 };
 
 typedef TileCfg<128, 128, 2, 2> Tile128x128;
@@ -80,9 +81,10 @@ typedef TileCfg<64, 128, 2, 2> Tile64x128;
 typedef TileCfg<128, 64, 2, 2> Tile128x64;
 typedef SkinnyCfg<1, 4> Skinny16;
 typedef SkinnyCfg<2, 4> Skinny32;
-typedef PipeCfg<2, 2, 4, 2, 3> Pipe256x128;
-typedef PipeCfg<2, 2, 2, 4, 3> Pipe128x256;
-typedef PipeCfg<4, 2, 2, 4, 2> Pipe256x256;    // 8 waves, wave tile 64 x 128
+typedef PipeCfg<2, 2, 4, 2, 3, 2, true> Pipe256x128;  // 4 waves, wave tile 128 x 64, register double buffering
+typedef PipeCfg<2, 2, 2, 4, 3, 2, true> Pipe128x256;  // 4 waves, wave tile 64 x 128
+typedef PipeCfg<4, 2, 2, 4, 2, 1> Pipe256x256;  // 8 waves, wave tile 64 x 128
+typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256p2;  // same, scale FMAs pipelined inside the wave
 typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
 
 constexpr int kMaxDevices = 64;
@@ -193,6 +195,7 @@ void tile_dims(int variant, int* bm, int* bn) {
       *bm = 128, *bn = 256;
       break;
     case kVarPipe256x256:
+    case kVarPipe256x256p2:
       *bm = 256, *bn = 256;
       break;
     default:
@@ -201,7 +204,7 @@ void tile_dims(int variant, int* bm, int* bn) {
 }
 
 bool is_skinny(int v) { return v == kVarSkinny16 || v == kVarSkinny32; }
-bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe128x256w8; }
+bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe256x256p2; }
 
 // Largest split count (<= limit) whose slices still hold `min_kb` K blocks each.
 int pick_splitk(int64_t units, int kblocks, int cus, int waves_per_unit, int min_kb, int limit) {
@@ -233,7 +236,7 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
   if (K % 16 != 0) v = kVarExact;
   if (is_pipelined(v) && (K % kScaleBlock != 0 || K == 0)) v = kVarTile128x128;  // DMA path moves whole K blocks
   if (v == kVarPipe256x128 && mode == kContiguous) v = kVarPipe128x256;       // a tile must not straddle experts
-  if (v == kVarPipe256x256 && mode == kContiguous) v = kVarPipe128x256w8;
+  if ((v == kVarPipe256x256 || v == kVarPipe256x256p2) && mode == kContiguous) v = kVarPipe128x256w8;
   if (is_skinny(v) && (mode != kDense || M > (v == kVarSkinny16 ? 16 : 32))) v = kVarTile128x128;
   if (v == kVarExact && mode != kDense) v = kVarTile128x128;
   pl.variant = v;
@@ -389,6 +392,8 @@ int run(const Problem& pr) {
         e = launch_pipelined_mode<Pipe128x256>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe256x256)
         e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarPipe256x256p2)
+        e = launch_pipelined_mode<Pipe256x256p2>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe128x256w8)
         e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarTile64x128)

@@ -10,8 +10,14 @@
 // Arithmetic: fp8_gemm_kernel of the reference (dlblas/kernels/fp8_gemm.py:49-60).  Requires K % 128 == 0.
 #pragma once
 
+#include <type_traits>
+
 #include "fp8_gemm_common.h"
 #include "fp8_gemm_tiled.h"  // xcd_remap
+
+#ifndef DLB_EXP
+#define DLB_EXP 0  // tuning builds set bits to cut pieces out of the K loop and time what is left (results are wrong)
+#endif
 
 namespace dlb {
 
@@ -74,9 +80,14 @@ __device__ __forceinline__ void wait_vmcnt() {
 // for later stages stay in flight across it; the caller waits for the group it needs with wait_vmcnt first.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_>
+// PARTS_: 2 = the scale FMAs of a fragment run under the MFMAs of the NEXT fragment of the same wave (two partial
+// accumulators); 1 = they follow their own MFMAs and overlap with the other wave of the SIMD instead (16 fewer VGPRs).
+// PREFETCH_: true (one wave per SIMD, 512 registers) = every fragment of the NEXT K step is read into a second
+// register set while the current step computes, so no MFMA of a step waits for LDS.
+template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_, int PARTS_ = 2, bool PREFETCH_ = false>
 struct PipeCfg {
-  static constexpr int WGM = WGM_, WGN = WGN_, MF = MF_, NF = NF_, STAGES = STAGES_;
+  static constexpr int WGM = WGM_, WGN = WGN_, MF = MF_, NF = NF_, STAGES = STAGES_, PARTS = PARTS_;
+  static constexpr bool PREFETCH = PREFETCH_;
   static constexpr int WAVES = WGM * WGN;
   static constexpr int NT = WAVES * 64;
   static constexpr int BM = WGM * MF * 32;
@@ -86,10 +97,11 @@ struct PipeCfg {
   static constexpr int S_INST = (BM + NT - 1) / NT;  // 4-byte DMA instructions per wave for the a_s slice
   static constexpr int A_BYTES = BM * kScaleBlock;
   static constexpr int B_BYTES = BN * kScaleBlock;
-  static constexpr int S_BYTES = S_INST * NT * 4;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + S_BYTES;
+  static constexpr int S_BYTES = S_INST * NT * 4;  // activation scales of the tile rows for one K block
+  static constexpr int W_BYTES = NT * 4;           // weight scale of each wave's n block, one copy per lane
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + S_BYTES + W_BYTES;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-  static constexpr int LOADS_PER_STAGE = A_INST + B_INST + S_INST;  // vmcnt units per wave and stage
+  static constexpr int LOADS_PER_STAGE = A_INST + B_INST + S_INST + 1;  // vmcnt units per wave and stage
   static_assert(BM % (8 * WAVES) == 0 && BN % (8 * WAVES) == 0, "tile rows must divide over the DMA instructions");
   static_assert(NF * 32 <= 128 && 128 % (NF * 32) == 0, "a wave's n span must stay inside one 128-wide scale block");
   static_assert(LOADS_PER_STAGE * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
@@ -181,14 +193,16 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
       const uint8_t* ag = a_tile + static_cast<int64_t>(kb) * kScaleBlock;
       const uint8_t* bg = b_tile + static_cast<int64_t>(kb) * kScaleBlock;
       const uint8_t* sg = reinterpret_cast<const uint8_t*>(as_tile + static_cast<int64_t>(kb) * p.as_sk);
+      int row0 = dma_row;
+      asm volatile("" : "+v"(row0));  // keeps the per-instruction offsets out of loop-invariant registers
 #pragma unroll
       for (int j = 0; j < Cfg::A_INST; ++j) {
-        const uint32_t off = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, a_last)) * uK + dma_chunk;
+        const uint32_t off = static_cast<uint32_t>(min(row0 + 8 * j * WAVES, a_last)) * uK + dma_chunk;
         dma_16(ag, off, sbase + (j * WAVES + wave) * 1024);
       }
 #pragma unroll
       for (int j = 0; j < Cfg::B_INST; ++j) {
-        const uint32_t off = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, b_last)) * uK + dma_chunk;
+        const uint32_t off = static_cast<uint32_t>(min(row0 + 8 * j * WAVES, b_last)) * uK + dma_chunk;
         dma_16(bg, off, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
       }
 #pragma unroll
@@ -197,6 +211,9 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
         const uint32_t off = static_cast<uint32_t>(min(row, a_last)) * static_cast<uint32_t>(p.as_sm) * 4u;
         dma_4(sg, off, sbase + Cfg::A_BYTES + Cfg::B_BYTES + (j * WAVES + wave) * 256);
       }
+      // every lane of the wave fetches the same weight scale b_s[n block of this wave][kb] into its own LDS slot
+      dma_4(reinterpret_cast<const uint8_t*>(bs_row + kb), 0u,
+            sbase + Cfg::A_BYTES + Cfg::B_BYTES + Cfg::S_BYTES + wave * 256);
     };
 
     v16f acc[MF][NF];
@@ -207,105 +224,215 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
 #pragma unroll
         for (int t = 0; t < 16; ++t) acc[mi][ni][t] = 0.f;
 
+    // ---- K loop ---------------------------------------------------------------------------------------------
+    // One operand's fragments are held in registers for the whole K step ("held": the one with fewer fragments),
+    // the other's are streamed past them one fragment at a time.  Tiles are visited streamed-major.  Registers
+    // are reloaded in place as soon as the last MFMA that reads them has been issued, and the single barrier of a
+    // K step sits before the tiles of the LAST streamed fragment: by then every LDS read of the current stage
+    // has returned, so the stage can be handed to the DMA, and the first fragments of the next stage are fetched
+    // while those last tiles run on the matrix pipe.  The step body is branch-free (the last steps are peeled
+    // through template flags) so that the scheduling fences inside it hold.
+    constexpr bool kHoldX = MF <= NF;          // hold activations (x), stream weights (w); else the reverse
+    constexpr int H = kHoldX ? MF : NF;        // held fragments
+    constexpr int S = kHoldX ? NF : MF;        // streamed fragments
+    constexpr int T = H * S;
+    constexpr int kFragBytes = 32 * kScaleBlock;
     const int nk = p.kblocks;
-    __syncthreads();  // the previous tile's readers are done with the ring
+    const int held0 = (kHoldX ? wm0 : Cfg::BM + wn0) * kScaleBlock;      // byte offset of held fragment 0 in a stage
+    const int strm0 = (kHoldX ? Cfg::BM + wn0 : wm0) * kScaleBlock;
+    constexpr int kScaleOff = Cfg::A_BYTES + Cfg::B_BYTES;
+    constexpr int kWScaleOff = kScaleOff + Cfg::S_BYTES;
+
+    __syncthreads();  // the previous tile's readers and DMA groups are done with the ring
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s)
-      if (s < nk) issue_stage(s, s);
+    for (int s = 0; s < STAGES; ++s) issue_stage(min(s, nk - 1), s);
+    if (STAGES >= 3)
+      wait_vmcnt<(STAGES - 1) * Cfg::LOADS_PER_STAGE>();
+    else
+      wait_vmcnt<Cfg::LOADS_PER_STAGE>();
+    lds_barrier();
 
-    // weight scales of this wave's n block: 64 K blocks per refill, one per lane, picked out with v_readlane
-    float bs_cache = 0.f;
-    constexpr int T = MF * NF;
-    int stage = 0;
-    for (int kb = 0; kb < nk; ++kb) {
-      if ((kb & 63) == 0) {
-        // refill the scale cache; the explicit drain keeps the compiler from waiting on this load (and with it
-        // on every DMA group in flight) at each later use
-        bs_cache = bs_row[min(kb + lane, nk - 1)];
-        wait_vmcnt<0>();
-        asm volatile("" : "+v"(bs_cache));
-      }
-      // stage kb's DMA is the oldest group in flight; at most STAGES - 2 younger groups may stay outstanding
-      const int younger = min(nk - 1 - kb, STAGES - 2);
-      if (younger >= 2)
-        wait_vmcnt<2 * Cfg::LOADS_PER_STAGE>();
-      else if (younger == 1)
-        wait_vmcnt<Cfg::LOADS_PER_STAGE>();
-      else
-        wait_vmcnt<0>();
-      lds_barrier();
-      if (kb + STAGES - 1 < nk) {
-        int fill = stage + STAGES - 1;
-        if (fill >= STAGES) fill -= STAGES;
-        issue_stage(kb + STAGES - 1, fill);
-      }
-
-      const int a_frag0 = stage * Cfg::STAGE_BYTES + wm0 * kScaleBlock;                 // wave-uniform byte offsets
-      const int b_frag0 = stage * Cfg::STAGE_BYTES + Cfg::A_BYTES + wn0 * kScaleBlock;
-      const float* sS = reinterpret_cast<const float*>(smem + stage * Cfg::STAGE_BYTES + Cfg::A_BYTES + Cfg::B_BYTES);
-      const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bs_cache), kb & 63));
-      constexpr int kFragBytes = 32 * kScaleBlock;
-
-      float sc[MF];
-#pragma unroll
-      for (int mi = 0; mi < MF; ++mi) sc[mi] = sS[wm0 + mi * 32 + l32] * sb;
-
-      // The scale FMAs of a fragment are issued after the MFMAs of the next one so that they run under them.
+    if constexpr (Cfg::PREFETCH) {
+      // ---- full register double buffering (one wave per SIMD) ------------------------------------------------
+      v8i xr[2][MF][2];
+      v8i wr[2][NF][2];
+      float scb[2][MF];
+      float sc_last = 0.f;
       v16f part[2];
-      if (MF >= NF) {
-        // keep the wave's weight fragments in registers, stream the activation fragments past them
-        v8i wf[NF][2];
-        v8i xf[2];
 #pragma unroll
-        for (int ni = 0; ni < NF; ++ni) {
-          wf[ni][0] = lds_read_frag32(smem, b_frag0 + ni * kFragBytes, lc, 0);
-          wf[ni][1] = lds_read_frag32(smem, b_frag0 + ni * kFragBytes, lc, 1);
-        }
-        xf[0] = lds_read_frag32(smem, a_frag0, lc, 0);
-        xf[1] = lds_read_frag32(smem, a_frag0, lc, 1);
+      for (int u = 0; u < 16; ++u) part[0][u] = part[1][u] = 0.f;
+      const int x0 = wm0 * kScaleBlock;
+      const int w0 = (Cfg::BM + wn0) * kScaleBlock;
+      auto load_scales = [&](int base, float (&dst)[MF]) {
+        const float sb = *reinterpret_cast<const float*>(smem + base + kWScaleOff + tid * 4);
+        const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
+#pragma unroll
+        for (int mi = 0; mi < MF; ++mi) dst[mi] = sS[wm0 + mi * 32 + l32] * sb;
+      };
+      // half-fragment q of a stage: q < 2 MF -> activation fragment q / 2, K half q % 2; else weight fragment
+      constexpr int kHalves = 2 * (MF + NF);
+      constexpr int kPerTile = (kHalves + (MF * NF) - 2) / (MF * NF - 1);  // spread over the first T - 1 tiles
+      load_scales(0, scb[0]);
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) {
+        xr[0][mi][0] = lds_read_frag32(smem, x0 + mi * kFragBytes, lc, 0);
+        xr[0][mi][1] = lds_read_frag32(smem, x0 + mi * kFragBytes, lc, 1);
+      }
+#pragma unroll
+      for (int ni = 0; ni < NF; ++ni) {
+        wr[0][ni][0] = lds_read_frag32(smem, w0 + ni * kFragBytes, lc, 0);
+        wr[0][ni][1] = lds_read_frag32(smem, w0 + ni * kFragBytes, lc, 1);
+      }
+
+      // Every step is the same code: a step always hands its stage to the DMA (past the end of K the DMA re-reads
+      // the last block into a stage nobody reads) and always prefetches "the next stage" (garbage after the last
+      // one, never used), so exactly STAGES - 1 DMA groups are in flight at every barrier and nothing is peeled.
+      auto k_step = [&](auto buf_tag, int kb, int stage) __attribute__((always_inline)) {
+        constexpr int B = decltype(buf_tag)::value;
+        const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+        const int nxt_base = next_stage * Cfg::STAGE_BYTES;
+        // every wave holds this stage's fragments in registers and has its share of the next stage in LDS
+        wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
+        lds_barrier();
+        issue_stage(min(kb + STAGES, nk - 1), stage);
 #pragma unroll
         for (int t = 0; t < T; ++t) {
           const int mi = t / NF, ni = t % NF;
+          __builtin_amdgcn_sched_barrier(0);
           v16f z;
 #pragma unroll
           for (int u = 0; u < 16; ++u) z[u] = 0.f;
-          z = mfma_32x32x64_e4m3(wf[ni][0], xf[0], z);
-          part[t & 1] = mfma_32x32x64_e4m3(wf[ni][1], xf[1], z);
-          if (ni == NF - 1 && mi + 1 < MF) {  // last use of this activation fragment has been issued: reload in place
-            xf[0] = lds_read_frag32(smem, a_frag0 + (mi + 1) * kFragBytes, lc, 0);
-            xf[1] = lds_read_frag32(smem, a_frag0 + (mi + 1) * kFragBytes, lc, 1);
+          z = mfma_32x32x64_e4m3(wr[B][ni][0], xr[B][mi][0], z);
+          part[t & 1] = mfma_32x32x64_e4m3(wr[B][ni][1], xr[B][mi][1], z);
+          __builtin_amdgcn_sched_barrier(0);
+          if (t == 0) load_scales(nxt_base, scb[B ^ 1]);
+#pragma unroll
+          for (int q = t * kPerTile; q < (t + 1) * kPerTile && q < kHalves; ++q) {
+            if (q < 2 * MF)
+              xr[B ^ 1][q / 2][q % 2] = lds_read_frag32(smem, nxt_base + x0 + (q / 2) * kFragBytes, lc, q % 2);
+            else
+              wr[B ^ 1][(q - 2 * MF) / 2][q % 2] =
+                  lds_read_frag32(smem, nxt_base + w0 + ((q - 2 * MF) / 2) * kFragBytes, lc, q % 2);
           }
-          if (t > 0) acc[(t - 1) / NF][(t - 1) % NF] += part[(t - 1) & 1] * sc[(t - 1) / NF];
+          __builtin_amdgcn_sched_barrier(0);
+          if (t == 0)
+            acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc_last;  // last tile of the previous K step
+          else
+            acc[(t - 1) / NF][(t - 1) % NF] += part[(t - 1) & 1] * scb[B][(t - 1) / NF];
         }
-        acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc[MF - 1];
-      } else {
-        // fewer activation fragments than weight fragments: keep the activations, stream the weights
-        v8i xf[MF][2];
-        v8i wf[2];
-#pragma unroll
-        for (int mi = 0; mi < MF; ++mi) {
-          xf[mi][0] = lds_read_frag32(smem, a_frag0 + mi * kFragBytes, lc, 0);
-          xf[mi][1] = lds_read_frag32(smem, a_frag0 + mi * kFragBytes, lc, 1);
-        }
-        wf[0] = lds_read_frag32(smem, b_frag0, lc, 0);
-        wf[1] = lds_read_frag32(smem, b_frag0, lc, 1);
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-          const int ni = t / MF, mi = t % MF;
-          v16f z;
-#pragma unroll
-          for (int u = 0; u < 16; ++u) z[u] = 0.f;
-          z = mfma_32x32x64_e4m3(wf[0], xf[mi][0], z);
-          part[t & 1] = mfma_32x32x64_e4m3(wf[1], xf[mi][1], z);
-          if (mi == MF - 1 && ni + 1 < NF) {  // last use of this weight fragment has been issued: reload in place
-            wf[0] = lds_read_frag32(smem, b_frag0 + (ni + 1) * kFragBytes, lc, 0);
-            wf[1] = lds_read_frag32(smem, b_frag0 + (ni + 1) * kFragBytes, lc, 1);
-          }
-          if (t > 0) acc[(t - 1) % MF][(t - 1) / MF] += part[(t - 1) & 1] * sc[(t - 1) % MF];
-        }
-        acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc[MF - 1];
+        sc_last = scb[B][MF - 1];
+      };
+      typedef std::integral_constant<int, 0> B0;
+      typedef std::integral_constant<int, 1> B1;
+      int stage = 0;
+      int kb = 0;
+      for (; kb + 1 < nk; kb += 2) {
+        k_step(B0{}, kb, stage);
+        stage = stage + 1 == STAGES ? 0 : stage + 1;
+        k_step(B1{}, kb + 1, stage);
+        stage = stage + 1 == STAGES ? 0 : stage + 1;
       }
+      if (kb < nk) k_step(B0{}, kb, stage);
+      acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc_last;
+      wait_vmcnt<0>();  // the trailing re-read groups must not land in the next tile's ring
+    } else {
+    v8i hf[H][2];
+    v8i sf[2];
+    float sc[MF];
+    float sc_last = 0.f;
+    v16f part[2];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) part[0][u] = part[1][u] = 0.f;
+
+    auto load_scales = [&](int base, float (&dst)[MF]) {
+      const float sb = *reinterpret_cast<const float*>(smem + base + kWScaleOff + tid * 4);
+      const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) dst[mi] = sS[wm0 + mi * 32 + l32] * sb;
+    };
+    load_scales(0, sc);
+#pragma unroll
+    for (int hi = 0; hi < H; ++hi) {
+      hf[hi][0] = lds_read_frag32(smem, held0 + hi * kFragBytes, lc, 0);
+      hf[hi][1] = lds_read_frag32(smem, held0 + hi * kFragBytes, lc, 1);
+    }
+    sf[0] = lds_read_frag32(smem, strm0, lc, 0);
+    sf[1] = lds_read_frag32(smem, strm0, lc, 1);
+
+    // One K step; every step is the same code (see the note in the register-double-buffered path above).
+    auto k_step = [&](int kb, int stage) __attribute__((always_inline)) {
+      const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+      const int cur_base = stage * Cfg::STAGE_BYTES;
+      const int nxt_base = next_stage * Cfg::STAGE_BYTES;
+      float sc_next[MF];
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        const int si = t / H, hi = t % H;
+        if (si == S - 1 && hi == 0) {
+          // every LDS read of this stage has been issued and the barrier waits for their return: hand it over
+          if (!(DLB_EXP & 8)) {
+            wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
+            lds_barrier();
+          }
+          if (!(DLB_EXP & 1)) issue_stage(min(kb + STAGES, nk - 1), stage);
+        }
+        // The scheduling fences pin the order MFMA pair -> reloads -> scale FMAs; without them the compiler
+        // hoists the reloads above the MFMAs into fresh registers and the kernel spills.
+        __builtin_amdgcn_sched_barrier(0);
+        v16f z;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) z[u] = 0.f;
+        constexpr int kSlot = Cfg::PARTS == 2 ? 1 : 0;
+        if (kHoldX) {
+          z = mfma_32x32x64_e4m3(sf[0], hf[hi][0], z);
+          part[t & kSlot] = mfma_32x32x64_e4m3(sf[1], hf[hi][1], z);
+        } else {
+          z = mfma_32x32x64_e4m3(hf[hi][0], sf[0], z);
+          part[t & kSlot] = mfma_32x32x64_e4m3(hf[hi][1], sf[1], z);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // in-place reloads: the MFMAs above were the last readers of these registers
+        if (hi == H - 1 && si + 1 < S && !(DLB_EXP & 4)) {
+          sf[0] = lds_read_frag32(smem, cur_base + strm0 + (si + 1) * kFragBytes, lc, 0);
+          sf[1] = lds_read_frag32(smem, cur_base + strm0 + (si + 1) * kFragBytes, lc, 1);
+        }
+        if (si == S - 1 && !(DLB_EXP & 4)) {
+          hf[hi][0] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 0);
+          hf[hi][1] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 1);
+          if (hi == 0) load_scales(nxt_base, sc_next);
+          if (hi == H - 1) {
+            sf[0] = lds_read_frag32(smem, nxt_base + strm0, lc, 0);
+            sf[1] = lds_read_frag32(smem, nxt_base + strm0, lc, 1);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (DLB_EXP & 2) {
+          const int mi = kHoldX ? hi : si, ni = kHoldX ? si : hi;
+          acc[mi][ni][0] += part[t & kSlot][t & 15];
+        } else if (Cfg::PARTS == 1) {
+          // scale-and-accumulate this tile; the other wave of the SIMD owns the matrix pipe meanwhile
+          const int mi = kHoldX ? hi : si, ni = kHoldX ? si : hi;
+          acc[mi][ni] += part[0] * sc[mi];
+        } else if (t == 0) {
+          // scale-and-accumulate the previous tile while this tile's MFMAs run
+          acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc_last;  // last tile of the previous K step (zero at kb = 0)
+        } else {
+          const int pt = t - 1;
+          const int pmi = kHoldX ? pt % H : pt / H, pni = kHoldX ? pt / H : pt % H;
+          acc[pmi][pni] += part[pt & 1] * sc[pmi];
+        }
+      }
+      sc_last = sc[MF - 1];
+#pragma unroll
+      for (int m2 = 0; m2 < MF; ++m2) sc[m2] = sc_next[m2];
+    };
+    int stage = 0;
+    for (int kb = 0; kb < nk; ++kb) {
+      k_step(kb, stage);
       stage = stage + 1 == STAGES ? 0 : stage + 1;
+    }
+    if (Cfg::PARTS == 2) acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc_last;
+    wait_vmcnt<0>();  // the trailing re-read groups must not land in the next tile's ring
     }
 
     // epilogue: lane holds c[m0 + wm0 + 32 mi + (lane & 31)][n0 + wn0 + 32 ni + 8 u + 4 (lane >> 5) + 0..3], u = 0..3
