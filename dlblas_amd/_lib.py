@@ -33,7 +33,7 @@ SYMBOLS = {
     'dlb_fp8_gemm_grouped_masked':
     (ctypes.c_int, [_c_vp] * 6 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 3 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
-    'dlb_fp8_gemm_force_splitk': (ctypes.c_int, [ctypes.c_int]),
+    'dlb_fp8_gemm_tune': (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
 }
 
@@ -119,9 +119,16 @@ def force_variant(name_or_id) -> None:
     check(lib.dlb_fp8_gemm_force_variant(int(name_or_id)))
 
 
+KNOBS = {'splitk': 0, 'skinny_waves': 1, 'skinny_unroll': 2, 'skinny_nfrags': 3, 'group_m': 4}
+
+
+def tune(knob: str, value) -> None:
+    """Set a tuning knob for later calls from this thread (None or 0: back to the heuristic)."""
+    check(load().dlb_fp8_gemm_tune(KNOBS[knob], int(value or 0)))
+
+
 def force_splitk(splitk) -> None:
-    """Pin the number of K splits of later dense calls from this thread (None or 0: heuristic)."""
-    check(load().dlb_fp8_gemm_force_splitk(int(splitk or 0)))
+    tune('splitk', splitk)
 
 
 def out_code(dtype: torch.dtype) -> int:

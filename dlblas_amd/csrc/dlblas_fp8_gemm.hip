@@ -47,7 +47,8 @@ namespace {
 
 thread_local char g_err[256] = "";
 thread_local int g_forced_variant = -1;
-thread_local int g_forced_splitk = 0;
+enum Knob : int { kKnobSplitK = 0, kKnobSkinnyWaves, kKnobSkinnyUnroll, kKnobSkinnyNFrags, kKnobGroupM, kKnobCount };
+thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0};
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -64,27 +65,25 @@ enum Variant : int {
   kVarTile128x64,
   kVarSkinny16,
   kVarSkinny32,
+  kVarSkinny64,
+  kVarSkinny128,
   kVarPipe256x128,
   kVarPipe128x256,
   kVarPipe256x256,
   kVarPipe128x256w8,
-  kVarPipe256x256p2,
   kVarCount
 };
 
 const char* const kVariantNames[kVarCount] = {
-    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8", "pipe256x256p2",
+    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "skinny64", "skinny128", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8",
 };
 
 typedef TileCfg<128, 128, 2, 2> Tile128x128;
 typedef TileCfg<64, 128, 2, 2> Tile64x128;
 typedef TileCfg<128, 64, 2, 2> Tile128x64;
-typedef SkinnyCfg<1, 4> Skinny16;
-typedef SkinnyCfg<2, 4> Skinny32;
 typedef PipeCfg<2, 2, 4, 2, 3, 2, true> Pipe256x128;  // 4 waves, wave tile 128 x 64, register double buffering
 typedef PipeCfg<2, 2, 2, 4, 3, 2, true> Pipe128x256;  // 4 waves, wave tile 64 x 128
-typedef PipeCfg<4, 2, 2, 4, 2, 1> Pipe256x256;  // 8 waves, wave tile 64 x 128
-typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256p2;  // same, scale FMAs pipelined inside the wave
+typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256;  // 8 waves, wave tile 64 x 128
 typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
 
 constexpr int kMaxDevices = 64;
@@ -160,9 +159,54 @@ hipError_t launch_pipelined_mode(int mode, const Args& args, int grid, int dev, 
 }
 
 template <class Cfg>
-hipError_t launch_skinny(const Args& args, hipStream_t stream) {
-  hipLaunchKernelGGL(fp8_gemm_skinny_kernel<Cfg>, dim3(args.tiles_n * args.splitk), dim3(Cfg::NT), 0, stream, args);
+hipError_t launch_skinny_cfg(const Args& args, int dev, hipStream_t stream) {
+  static std::atomic<unsigned long long> lds_done{0}, lds_done_tail{0};
+  const bool ktail = args.K % kScaleBlock != 0;
+  auto kernel = ktail ? fp8_gemm_skinny_kernel<Cfg, true> : fp8_gemm_skinny_kernel<Cfg, false>;
+  hipError_t e = ensure_lds(kernel, Cfg::RED_BYTES, dev, ktail ? &lds_done_tail : &lds_done);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kernel, dim3(args.tiles_n), dim3(Cfg::NT), Cfg::RED_BYTES, stream, args);
   return hipGetLastError();
+}
+
+// Skinny kernel instances: MF in {1, 2}, (waves, unroll) in a small set, n fragments in {1, 2}.
+template <int MF, int NFS>
+hipError_t launch_skinny_wu(int waves, int unroll, const Args& args, int dev, hipStream_t stream) {
+  if (waves >= 16) {
+    if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 16, 4, NFS>>(args, dev, stream);
+    if (unroll >= 2) return launch_skinny_cfg<SkinnyCfg<MF, 16, 2, NFS>>(args, dev, stream);
+    return launch_skinny_cfg<SkinnyCfg<MF, 16, 1, NFS>>(args, dev, stream);
+  }
+  if (waves >= 8) {
+    if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 8, 4, NFS>>(args, dev, stream);
+    if (unroll >= 2) return launch_skinny_cfg<SkinnyCfg<MF, 8, 2, NFS>>(args, dev, stream);
+    return launch_skinny_cfg<SkinnyCfg<MF, 8, 1, NFS>>(args, dev, stream);
+  }
+  if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 4, 4, NFS>>(args, dev, stream);
+  return launch_skinny_cfg<SkinnyCfg<MF, 4, 2, NFS>>(args, dev, stream);
+}
+
+// Large activation blocks (M up to 64 / 128) keep to one K block in flight per wave: their fragments fill the registers.
+template <int MF, int NFS>
+hipError_t launch_skinny_big(int waves, const Args& args, int dev, hipStream_t stream) {
+  if (waves >= 16) return launch_skinny_cfg<SkinnyCfg<MF, 16, 1, NFS>>(args, dev, stream);
+  if (waves >= 8) return launch_skinny_cfg<SkinnyCfg<MF, 8, 1, NFS>>(args, dev, stream);
+  return launch_skinny_cfg<SkinnyCfg<MF, 4, 1, NFS>>(args, dev, stream);
+}
+
+hipError_t launch_skinny(int mf, int nfs, int waves, int unroll, const Args& args, int dev, hipStream_t stream) {
+  switch (mf) {
+    case 1:
+      return nfs == 2 ? launch_skinny_wu<1, 2>(waves, unroll, args, dev, stream)
+                      : launch_skinny_wu<1, 1>(waves, unroll, args, dev, stream);
+    case 2:
+      return nfs == 2 ? launch_skinny_wu<2, 2>(waves, unroll, args, dev, stream)
+                      : launch_skinny_wu<2, 1>(waves, unroll, args, dev, stream);
+    case 4:
+      return nfs == 2 ? launch_skinny_big<4, 2>(waves, args, dev, stream) : launch_skinny_big<4, 1>(waves, args, dev, stream);
+    default:
+      return nfs == 2 ? launch_skinny_big<8, 2>(waves, args, dev, stream) : launch_skinny_big<8, 1>(waves, args, dev, stream);
+  }
 }
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -171,6 +215,7 @@ struct Plan {
   int variant;
   int bm, bn;
   int splitk;
+  int sk_waves, sk_unroll, sk_nfrags;  // skinny kernel shape
 };
 
 void tile_dims(int variant, int* bm, int* bn) {
@@ -187,6 +232,12 @@ void tile_dims(int variant, int* bm, int* bn) {
     case kVarSkinny32:
       *bm = 32, *bn = 16;
       break;
+    case kVarSkinny64:
+      *bm = 64, *bn = 16;
+      break;
+    case kVarSkinny128:
+      *bm = 128, *bn = 16;
+      break;
     case kVarPipe256x128:
       *bm = 256, *bn = 128;
       break;
@@ -195,7 +246,6 @@ void tile_dims(int variant, int* bm, int* bn) {
       *bm = 128, *bn = 256;
       break;
     case kVarPipe256x256:
-    case kVarPipe256x256p2:
       *bm = 256, *bn = 256;
       break;
     default:
@@ -203,8 +253,9 @@ void tile_dims(int variant, int* bm, int* bn) {
   }
 }
 
-bool is_skinny(int v) { return v == kVarSkinny16 || v == kVarSkinny32; }
-bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe256x256p2; }
+bool is_skinny(int v) { return v >= kVarSkinny16 && v <= kVarSkinny128; }
+int skinny_rows(int v) { return 16 << (v - kVarSkinny16); }
+bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe128x256w8; }
 
 // Largest split count (<= limit) whose slices still hold `min_kb` K blocks each.
 int pick_splitk(int64_t units, int kblocks, int cus, int waves_per_unit, int min_kb, int limit) {
@@ -218,39 +269,52 @@ int pick_splitk(int64_t units, int kblocks, int cus, int waves_per_unit, int min
 }
 
 Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes) {
-  Plan pl{kVarTile128x128, 128, 128, 1};
+  Plan pl{kVarTile128x128, 128, 128, 1, 4, 4, 1};
   const int kblocks = static_cast<int>(ceil_div(K, kScaleBlock));
   int v = g_forced_variant;
   if (v < 0) {
-    if (K % 16 != 0)
+    const bool whole_blocks = K > 0 && K % kScaleBlock == 0;
+    if (K % 16 != 0) {
       v = kVarExact;
-    else if (mode == kDense && M <= 16)
-      v = kVarSkinny16;
-    else if (mode == kDense && M <= 32)
-      v = kVarSkinny32;
-    else if (M <= 64 && mode != kContiguous)
-      v = kVarTile64x128;
-    else
-      v = kVarTile128x128;
+    } else if (mode == kDense && M <= 128) {
+      // decode: stream the weights once, K split over the waves of a workgroup
+      v = M <= 16 ? kVarSkinny16 : (M <= 32 ? kVarSkinny32 : (M <= 64 ? kVarSkinny64 : kVarSkinny128));
+    } else if (whole_blocks && mode == kDense) {
+      const int64_t t256 = ceil_div(M, 256) * ceil_div(N, 256);
+      const int64_t t128 = ceil_div(M, 128) * ceil_div(N, 256);
+      v = t256 * 2 >= cus ? kVarPipe256x256 : (t128 * 4 >= cus ? kVarPipe128x256w8 : kVarTile128x128);
+    } else if (whole_blocks) {
+      v = kVarPipe128x256w8;  // grouped: 128-row tiles never straddle two experts / waste at most 127 masked rows
+    } else {
+      v = (M <= 64 && mode != kContiguous) ? kVarTile64x128 : kVarTile128x128;
+    }
   }
   if (K % 16 != 0) v = kVarExact;
   if (is_pipelined(v) && (K % kScaleBlock != 0 || K == 0)) v = kVarTile128x128;  // DMA path moves whole K blocks
   if (v == kVarPipe256x128 && mode == kContiguous) v = kVarPipe128x256;       // a tile must not straddle experts
-  if ((v == kVarPipe256x256 || v == kVarPipe256x256p2) && mode == kContiguous) v = kVarPipe128x256w8;
-  if (is_skinny(v) && (mode != kDense || M > (v == kVarSkinny16 ? 16 : 32))) v = kVarTile128x128;
+  if (v == kVarPipe256x256 && mode == kContiguous) v = kVarPipe128x256w8;
+  if (is_skinny(v) && (mode != kDense || M > skinny_rows(v))) v = kVarTile128x128;
   if (v == kVarExact && mode != kDense) v = kVarTile128x128;
   pl.variant = v;
   tile_dims(v, &pl.bm, &pl.bn);
-  if (mode != kDense || v == kVarExact || kblocks < 2 || is_pipelined(v)) return pl;
+  if (mode != kDense || v == kVarExact || is_pipelined(v) || (kblocks < 2 && !is_skinny(v))) return pl;
 
   const int64_t tiles_n = ceil_div(N, pl.bn);
   const size_t avail = ws_bytes > DLB_WS_COUNTER_BYTES ? ws_bytes - DLB_WS_COUNTER_BYTES : 0;
   if (is_skinny(v)) {
-    if (tiles_n > DLB_WS_COUNTER_BYTES / 4) return pl;
-    int s = pick_splitk(tiles_n, kblocks, cus, 4, 4, 16);
-    const size_t per_split = static_cast<size_t>(tiles_n) * (pl.bm / 16) * 256 * sizeof(float);
-    while (s > 1 && per_split * s > avail) --s;
-    pl.splitk = s;
+    // K is split over the waves of a workgroup only.  Pick the wave count so that every wave has two or so K
+    // blocks and the unroll so that a wave issues all of its loads before its first MFMA.
+    int waves = kblocks >= 8 ? 8 : 4;
+    if (g_knob[kKnobSkinnyWaves] > 0) waves = g_knob[kKnobSkinnyWaves];
+    const int per_wave = static_cast<int>(ceil_div(kblocks, waves));
+    // measured on MI355X: one K block in flight per wave is as good as more once eight waves share a row block
+    int unroll = waves >= 8 ? 1 : (per_wave >= 3 ? 4 : 2);
+    if (g_knob[kKnobSkinnyUnroll] > 0) unroll = g_knob[kKnobSkinnyUnroll];
+    // two weight fragments per workgroup halve the activation re-reads, but only while the grid still covers the chip
+    int nfrags = ceil_div(N, 32) * 4 >= 3 * cus ? 2 : 1;
+    if (g_knob[kKnobSkinnyNFrags] > 0) nfrags = g_knob[kKnobSkinnyNFrags];
+    pl.sk_waves = waves, pl.sk_unroll = unroll, pl.sk_nfrags = nfrags >= 2 ? 2 : 1;
+    pl.bn = 16 * pl.sk_nfrags;
   } else {
     const int64_t tiles = ceil_div(M, pl.bm) * tiles_n;
     if (tiles > DLB_WS_COUNTER_BYTES / 4 || tiles * 2 > cus) return pl;
@@ -320,7 +384,9 @@ int run(const Problem& pr) {
   if (cus < 0) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
 
   Plan pl = make_plan(pr.mode, pr.rows, pr.N, pr.K, cus, pr.ws ? pr.ws_bytes : 0);
-  if (g_forced_splitk > 0 && pr.mode == kDense && pl.variant != kVarExact) pl.splitk = g_forced_splitk;
+  if (g_knob[kKnobSplitK] > 0 && pr.mode == kDense && pl.variant != kVarExact && !is_skinny(pl.variant) &&
+      !is_pipelined(pl.variant))
+    pl.splitk = g_knob[kKnobSplitK];
   if (pl.splitk > 1) {
     if (!pr.ws || pr.ws_bytes < DLB_WS_COUNTER_BYTES) pl.splitk = 1;
     if (misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
@@ -352,7 +418,7 @@ int run(const Problem& pr) {
   ar.splitk = pl.splitk;
   ar.kb_per_split = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, pl.splitk));
   ar.splitk = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, ar.kb_per_split));  // no empty splits
-  ar.group_m = 8;
+  ar.group_m = g_knob[kKnobGroupM] > 0 ? g_knob[kKnobGroupM] : 8;
   ar.out_f32 = pr.out_dtype == DLB_OUT_F32;
   const size_t esz = ar.out_f32 ? 4 : 2;
   ar.vec_store = (pr.N % 4 == 0) && !misaligned(pr.c, 4 * esz);
@@ -372,10 +438,16 @@ int run(const Problem& pr) {
       break;
     }
     case kVarSkinny16:
-      e = launch_skinny<Skinny16>(ar, pr.stream);
+      e = launch_skinny(1, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
       break;
     case kVarSkinny32:
-      e = launch_skinny<Skinny32>(ar, pr.stream);
+      e = launch_skinny(2, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
+      break;
+    case kVarSkinny64:
+      e = launch_skinny(4, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
+      break;
+    case kVarSkinny128:
+      e = launch_skinny(8, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
       break;
     default: {
       int64_t grid = tiles;
@@ -392,8 +464,6 @@ int run(const Problem& pr) {
         e = launch_pipelined_mode<Pipe128x256>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe256x256)
         e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g, dev, pr.stream);
-      else if (pl.variant == kVarPipe256x256p2)
-        e = launch_pipelined_mode<Pipe256x256p2>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe128x256w8)
         e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarTile64x128)
@@ -465,9 +535,10 @@ int dlb_fp8_gemm_force_variant(int variant) {
   return DLB_OK;
 }
 
-int dlb_fp8_gemm_force_splitk(int splitk) {
-  if (splitk < 0 || splitk > 64) return dlb::fail(DLB_ERR_BAD_SHAPE, "split count %d outside [0, 64]", splitk);
-  dlb::g_forced_splitk = splitk;
+int dlb_fp8_gemm_tune(int knob, int value) {
+  if (knob < 0 || knob >= dlb::kKnobCount) return dlb::fail(DLB_ERR_BAD_SHAPE, "unknown tuning knob %d", knob);
+  if (value < 0 || value > 1024) return dlb::fail(DLB_ERR_BAD_SHAPE, "tuning value %d outside [0, 1024]", value);
+  dlb::g_knob[knob] = value;
   return DLB_OK;
 }
 

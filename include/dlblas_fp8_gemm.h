@@ -149,10 +149,19 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
 int dlb_fp8_gemm_force_variant(int variant);
 
 /*
- * Tuning / test hook: force the number of K splits of the next dense calls FROM THIS THREAD (clamped to what the
- * workspace and K allow); 0 restores the heuristic.  Grouped calls never split K.
+ * Tuning / test hook: set knob `knob` for the next calls FROM THIS THREAD; value 0 restores the heuristic.
+ *   DLB_KNOB_SPLITK         K splits of the LDS-tiled dense kernels (clamped to what workspace and K allow)
+ *   DLB_KNOB_SKINNY_WAVES   waves per workgroup of the decode kernels (4, 8 or 16)
+ *   DLB_KNOB_SKINNY_UNROLL  K blocks a decode-kernel wave loads before its first MFMA (1, 2 or 4)
+ *   DLB_KNOB_SKINNY_NFRAGS  16-row weight fragments per decode workgroup (1 or 2)
+ *   DLB_KNOB_GROUP_M        m-tiles per L2 swizzle group of the tiled kernels
  */
-int dlb_fp8_gemm_force_splitk(int splitk);
+#define DLB_KNOB_SPLITK 0
+#define DLB_KNOB_SKINNY_WAVES 1
+#define DLB_KNOB_SKINNY_UNROLL 2
+#define DLB_KNOB_SKINNY_NFRAGS 3
+#define DLB_KNOB_GROUP_M 4
+int dlb_fp8_gemm_tune(int knob, int value);
 
 /* Name of kernel variant `variant`, or NULL beyond the last one. */
 const char* dlb_fp8_gemm_variant_name(int variant);
