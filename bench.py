@@ -31,6 +31,10 @@ WORKLOADS = {
     'decode_16x2112x7168': ('dense', 16, 2112, 7168),
     'cpu_case_64x512x1024': ('dense', 64, 512, 1024),
 }
+# measured after the timed region and reported under "other_workloads" (name: M, N, K)
+DECODE_SWEEP = [(m, n, k) for (n, k) in ((7168, 2048), (2112, 7168)) for m in (1, 16, 64, 128)]
+GROUPED_CONTIGUOUS = dict(G=32, tokens=8192, N=4096, K=7168)
+GROUPED_MASKED = dict(G=32, M_max=256, N=7168, K=2048)
 
 
 def log(msg):
@@ -127,34 +131,135 @@ def time_steps(launch, steps, warmup):
     return wall_ms / steps, start.elapsed_time(stop) / steps
 
 
-def cpu_baseline(kind, M, N, K, a_q, a_s, b_q, b_s, budget_s=15.0):
-    """The reference CPU path (dequantise to fp32, torch.matmul) timed on this host on a bounded row sample."""
+def cpu_baseline(kind, M, N, K, a_q, a_s, b_q, b_s, budget_s=12.0):
+    """The reference CPU path (dequantise both operands to fp32, torch.matmul, cast to bf16) timed on this host:
+    whole passes over a row sample of the workload, repeated until about `budget_s` seconds of CPU work are done."""
     import torch
 
     from oracle import fp8_block_gemm as orc
     a_q, a_s, b_q, b_s = a_q.cpu(), a_s.cpu(), b_q.cpu(), b_s.cpu()
-    probe_rows = min(M, 32)
-    t0 = time.perf_counter()
-    orc.dequant_ref(a_q[:probe_rows], a_s[:probe_rows], b_q, b_s, torch.bfloat16)
-    probe = time.perf_counter() - t0
-    # the weight dequantisation is a fixed cost; scale rows so that the whole sample takes about budget_s
-    t0 = time.perf_counter()
-    orc.dequant_ref(a_q[:1], a_s[:1], b_q, b_s, torch.bfloat16)
-    fixed = time.perf_counter() - t0
-    per_row = max((probe - fixed) / max(probe_rows - 1, 1), 1e-9)
-    rows = int(max(probe_rows, min(M, (budget_s - fixed) / per_row)))
+    rows = min(M, 1024)
     t0 = time.perf_counter()
     orc.dequant_ref(a_q[:rows], a_s[:rows], b_q, b_s, torch.bfloat16)
-    dt = time.perf_counter() - t0
+    first = time.perf_counter() - t0
+    if first < budget_s / 8 and rows < M:
+        rows = M
+    times = []
+    spent = 0.0
+    while spent < budget_s and len(times) < 50:
+        t0 = time.perf_counter()
+        orc.dequant_ref(a_q[:rows], a_s[:rows], b_q, b_s, torch.bfloat16)
+        times.append(time.perf_counter() - t0)
+        spent += times[-1]
+    times.sort()
+    dt = times[len(times) // 2]
     flops = 2.0 * rows * N * K
     return {
         'value': flops / dt / 1e12,
         'unit': 'TFLOP/s',
         'cores': torch.get_num_threads(),
         'kind': 'port',
-        'sample': f'first {rows} of {M} rows x N={N} x K={K} (dequantise both operands to fp32 + torch.matmul), '
-                  f'{dt:.1f} s',
+        'sample': f'first {rows} of {M} rows x N={N} x K={K}: dequantise both operands to fp32 + torch.matmul + bf16 '
+                  f'cast, median of {len(times)} passes ({spent:.1f} s of CPU work, {dt:.2f} s per pass)',
     }
+
+
+def time_call(fn, iters, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def decode_sweep(dev):
+    """HBM-bound shapes: 24 distinct weight copies in rotation (> 256 MB) so that reads come from HBM."""
+    import torch
+    rows = []
+    for (M, N, K) in DECODE_SWEEP:
+        a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=24)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        ms = time_call(DenseLauncher(a_q, a_s, ws, out), 480, 48)
+        nbytes = algorithmic_bytes(M, N, K)
+        rows.append({'workload': f'decode_{M}x{N}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
+                     'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'TFLOPs': 2.0 * M * N * K / ms / 1e9,
+                     'bytes': nbytes})
+        del a_q, a_s, ws, out
+    return rows
+
+
+def expert_weights(G, N, K, dev, seed):
+    import torch
+    g = torch.Generator(device=dev).manual_seed(seed)
+    qs, ss = [], []
+    for _ in range(G):
+        q, s = quantise_weight((torch.randn(N, K, device=dev, generator=g) * 0.02).to(torch.bfloat16))
+        qs.append(q)
+        ss.append(s)
+    return torch.stack(qs), torch.stack(ss)
+
+
+def grouped_workloads(dev):
+    """One GPU's expert share of the two MoE layouts; FLOPs count real tokens only, bytes count every operand once."""
+    import torch
+
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_contiguous, fp8_gemm_grouped_masked
+    rows = []
+    # expert-contiguous (prefill): per-expert counts from a seeded multinomial, padded to multiples of 128
+    c = GROUPED_CONTIGUOUS
+    G, N, K = c['G'], c['N'], c['K']
+    g = torch.Generator().manual_seed(20)
+    assign = torch.multinomial(torch.full((G, ), 1.0 / G), c['tokens'], replacement=True, generator=g)
+    counts = torch.bincount(assign, minlength=G)
+    padded = (counts + 127) // 128 * 128
+    M_sum = int(padded.sum())
+    m_indices = torch.repeat_interleave(torch.arange(G, dtype=torch.int32), padded).to(dev)
+    gd = torch.Generator(device=dev).manual_seed(21)
+    a_q, a_s = quantise_act(torch.randn(M_sum, K, device=dev, generator=gd).to(torch.bfloat16))
+    w_q, w_s = expert_weights(G, N, K, dev, 22)
+    out = torch.empty(M_sum, N, dtype=torch.bfloat16, device=dev)
+    ms = time_call(lambda: fp8_gemm_grouped_contiguous(a_q, a_s, w_q, w_s, out, m_indices), 20, 3)
+    flops = 2.0 * c['tokens'] * N * K
+    nbytes = M_sum * K + G * N * K + 4 * M_sum * (K // 128) + 4 * G * (N // 128) * (K // 128) + 2 * M_sum * N + 4 * M_sum
+    rows.append({'workload': f'grouped_contiguous_E{G}_T{c["tokens"]}_N{N}_K{K}', 'M_sum_padded': M_sum,
+                 'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9, 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS,
+                 'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS})
+    del a_q, a_s, w_q, w_s, out
+    # masked (decode): valid rows uniform in [0, M_max]
+    c = GROUPED_MASKED
+    G, M_max, N, K = c['G'], c['M_max'], c['N'], c['K']
+    masked_m = torch.randint(0, M_max + 1, (G, ), generator=torch.Generator().manual_seed(20), dtype=torch.int32)
+    a_q, a_s = quantise_act(torch.randn(G * M_max, K, device=dev, generator=gd).to(torch.bfloat16))
+    a_q, a_s = a_q.reshape(G, M_max, K), a_s.reshape(G, M_max, K // 128)
+    w_q, w_s = expert_weights(G, N, K, dev, 24)
+    out = torch.empty(G, M_max, N, dtype=torch.bfloat16, device=dev)
+    mm = masked_m.to(dev)
+    hint = int(masked_m.float().mean())
+    ms = time_call(lambda: fp8_gemm_grouped_masked(a_q, a_s, w_q, w_s, out, mm, hint), 20, 3)
+    valid = int(masked_m.sum())
+    flops = 2.0 * valid * N * K
+    nbytes = valid * K + G * N * K + 4 * valid * (K // 128) + 4 * G * (N // 128) * (K // 128) + 2 * valid * N + 4 * G
+    rows.append({'workload': f'grouped_masked_E{G}_Mmax{M_max}_N{N}_K{K}', 'valid_rows': valid,
+                 'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9, 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS,
+                 'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS})
+    return rows
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the dominant kernel from the rocprofv3 --pmc runs kept under profiles/ (None when
+    no counter run for this workload has been recorded)."""
+    path = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+    try:
+        with open(path) as fh:
+            return json.load(fh).get(workload, {}).get('bytes_per_launch')
+    except (OSError, ValueError):
+        return None
 
 
 def main():
@@ -165,7 +270,9 @@ def main():
     ap.add_argument('--workload', default='prefill_4096x7168x18432', choices=sorted(WORKLOADS))
     ap.add_argument('--variant', default=None, help='force a kernel variant (tuning)')
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--no-decode', action='store_true')
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='also run three 1 GiB device copies: the known-size kernel that HBM counters are scaled by')
+    ap.add_argument('--no-other', action='store_true', help='skip the decode sweep and the grouped workloads')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1', file=sys.stderr)
@@ -200,7 +307,7 @@ def main():
         roofline = {'bound': 'mfma', 'achieved': flops / (ev_ms * 1e-3) / 1e12, 'peak': PEAK_FP8_TFLOPS,
                     'unit': 'TFLOP/s'}
     roofline['frac'] = roofline['achieved'] / roofline['peak']
-    roofline['traffic'] = None
+    roofline['traffic'] = measured_traffic(args.workload)
     roofline['kernel_ms'] = ev_ms
 
     result = {
@@ -221,19 +328,24 @@ def main():
         'roofline': roofline,
     }
 
-    if not args.no_decode and not memory_bound:
-        dM, dN, dK = 16, 7168, 2048
-        log(f'decode M={dM} N={dN} K={dK}')
-        da_q, da_s, dws = make_inputs(dM, dN, dK, dev, weight_copies=24)
-        dout = torch.empty(dM, dN, dtype=torch.bfloat16, device=dev)
-        dl = DenseLauncher(da_q, da_s, dws, dout)
-        d_wall, d_ev = time_steps(dl, 480, 48)
-        db = algorithmic_bytes(dM, dN, dK)
-        result['decode'] = {
-            'workload': f'decode_{dM}x{dN}x{dK}', 'us_per_launch': d_ev * 1e3, 'GBps': db / (d_ev * 1e-3) / 1e9,
-            'frac_of_hbm_peak': db / (d_ev * 1e-3) / 1e9 / PEAK_HBM_GBS, 'bytes': db,
-            'note': '24 distinct weight copies in rotation (353 MB) so reads miss the 256 MB cache'
-        }
+    if not args.no_other:
+        log('decode sweep')
+        others = decode_sweep(dev)
+        m16 = next(r for r in others if r['workload'] == 'decode_16x7168x2048')
+        result['decode'] = {'workload': m16['workload'], 'us_per_launch': m16['us_per_launch'], 'GBps': m16['GBps'],
+                            'frac_of_hbm_peak': m16['frac_of_hbm_peak'], 'bytes': m16['bytes'],
+                            'note': '24 distinct weight copies in rotation (353 MB) so reads miss the 256 MB cache'}
+        log('grouped workloads')
+        others += grouped_workloads(dev)
+        result['other_workloads'] = others
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     if not args.no_cpu_baseline:
         log('cpu baseline')
