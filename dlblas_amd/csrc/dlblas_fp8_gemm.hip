@@ -428,6 +428,25 @@ int run(const Problem& pr) {
   }
 
   hipError_t e = hipSuccess;
+  if (is_pipelined(pl.variant) && pr.as_sk == 1 && pr.as_sm > 1 && ar.ws && kblocks > 1) {
+    // row-major activation scales: re-lay them rows-contiguous in the workspace first (a few microseconds) so the
+    // GEMM fetches 8 cache lines of scales per K step and tile instead of 256
+    const int64_t rows_pad = (pr.rows + 3) / 4 * 4;
+    const int64_t need = groups * kblocks * rows_pad * static_cast<int64_t>(sizeof(float));
+    if (static_cast<size_t>(need) + DLB_WS_COUNTER_BYTES <= pr.ws_bytes && rows_pad * kblocks < (1ll << 31)) {
+      const dim3 tgrid(static_cast<unsigned>(ceil_div(rows_pad, 32)), static_cast<unsigned>(ceil_div(kblocks, 32)),
+                       static_cast<unsigned>(pr.mode == kMasked ? groups : 1));
+      hipLaunchKernelGGL(fp8_scale_transpose_kernel, tgrid, dim3(256), 0, pr.stream, pr.a_s, ar.ws, static_cast<int>(pr.rows),
+                         static_cast<int>(kblocks), static_cast<int>(rows_pad), pr.mode == kMasked ? pr.as_sg : 0, pr.as_sm,
+                         pr.as_sk);
+      e = hipGetLastError();
+      if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "scale re-layout launch failed: %s", hipGetErrorString(e));
+      ar.a_s = ar.ws;
+      ar.as_sm = 1;
+      ar.as_sk = rows_pad;
+      ar.as_gs = kblocks * rows_pad;
+    }
+  }
   const int64_t tiles = static_cast<int64_t>(ar.tiles_m) * ar.tiles_n * ar.splitk;
   switch (pl.variant) {
     case kVarExact: {

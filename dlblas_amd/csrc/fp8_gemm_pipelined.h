@@ -107,6 +107,31 @@ struct PipeCfg {
   static_assert(LOADS_PER_STAGE * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
 };
 
+// Re-lays activation scales from [groups][rows][kblocks] (any strides) to [groups][kblocks][rows_pad], rows
+// contiguous, so that the GEMM's per-K-step fetch of one scale per tile row is a handful of full cache lines
+// instead of one line per row.  32 x 32 tiles through LDS keep both sides coalesced.  (The reference does the same
+// re-layout before its grouped GEMMs, dlblas/kernels/quant_dequant.py:42-83.)
+__global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* src, float* dst, int rows, int kblocks,
+                                                                  int rows_pad, int64_t s_g, int64_t s_m, int64_t s_k) {
+  __shared__ float tile[32][33];
+  const int g = blockIdx.z;
+  const int r0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const float* in = src + static_cast<int64_t>(g) * s_g;
+  float* out = dst + static_cast<int64_t>(g) * kblocks * rows_pad;
+#pragma unroll
+  for (int i = 0; i < 32; i += 8) {
+    const int r = r0 + ty + i, k = k0 + tx;
+    tile[ty + i][tx] = (r < rows && k < kblocks) ? in[static_cast<int64_t>(r) * s_m + static_cast<int64_t>(k) * s_k] : 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 32; i += 8) {
+    const int k = k0 + ty + i, r = r0 + tx;
+    if (k < kblocks && r < rows_pad) out[static_cast<int64_t>(k) * rows_pad + r] = tile[tx][ty + i];
+  }
+}
+
 template <class Cfg, int MODE>
 __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args p) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MF = Cfg::MF, NF = Cfg::NF, WAVES = Cfg::WAVES, STAGES = Cfg::STAGES;
