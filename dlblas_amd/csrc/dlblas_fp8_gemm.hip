@@ -3,6 +3,9 @@
 #include "../../include/dlblas_fp8_gemm.h"
 
 #include <atomic>
+#include <functional>
+#include <queue>
+#include <vector>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -71,11 +74,12 @@ enum Variant : int {
   kVarPipe128x256,
   kVarPipe256x256,
   kVarPipe128x256w8,
+  kVarPipe256mix,
   kVarCount
 };
 
 const char* const kVariantNames[kVarCount] = {
-    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "skinny64", "skinny128", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8",
+    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "skinny64", "skinny128", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8", "pipe256mix",
 };
 
 typedef TileCfg<128, 128, 2, 2> Tile128x128;
@@ -84,6 +88,7 @@ typedef TileCfg<128, 64, 2, 2> Tile128x64;
 typedef PipeCfg<2, 2, 4, 2, 3, 2, true> Pipe256x128;  // 4 waves, wave tile 128 x 64, register double buffering
 typedef PipeCfg<2, 2, 2, 4, 3, 2, true> Pipe128x256;  // 4 waves, wave tile 64 x 128
 typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256;  // 8 waves, wave tile 64 x 128
+typedef PipeCfg<4, 2, 2, 3, 2, 2> Pipe256x192;  // narrow tiles of the mixed-width launch
 typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
 
 constexpr int kMaxDevices = 64;
@@ -211,6 +216,46 @@ hipError_t launch_skinny(int mf, int nfs, int waves, int unroll, const Args& arg
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Makespan (in units of one 256 x 256 tile) of `ta` tiles of cost 1 followed by `tb` tiles of cost `cb`, handed
+// out in order, each to the worker that becomes free first.
+double mixed_makespan(int64_t ta, int64_t tb, double cb, int workers) {
+  std::priority_queue<double, std::vector<double>, std::greater<double>> free_at;
+  for (int i = 0; i < workers; ++i) free_at.push(0.0);
+  double end = 0.0;
+  for (int64_t t = 0; t < ta + tb; ++t) {
+    const double done = free_at.top() + (t < ta ? 1.0 : cb);
+    free_at.pop();
+    free_at.push(done);
+    if (done > end) end = done;
+  }
+  return end;
+}
+
+// Columns [0, n_split) in 256-wide tiles, the rest in 192-wide tiles; returns n_split (== N: no narrow region).
+int64_t pick_mixed_split(int64_t M, int64_t N, int cus) {
+  // the search simulates a few thousand tile hand-outs: remember the answers of the shapes seen by this thread
+  struct Memo { int64_t M, N; int cus; int64_t split; };
+  thread_local Memo memo[8] = {};
+  thread_local int memo_next = 0;
+  for (const Memo& m : memo)
+    if (m.M == M && m.N == N && m.cus == cus && m.M > 0) return m.split;
+  const int64_t tm = ceil_div(M, 256);
+  const double narrow_cost = 0.78;  // 192 / 256 of the work plus the fixed per-tile part
+  int64_t best_split = N;
+  double best = mixed_makespan(tm * ceil_div(N, 256), 0, narrow_cost, cus);
+  if (tm * ceil_div(N, 256) <= 16 * static_cast<int64_t>(cus)) {  // many rounds: the tail no longer matters
+    for (int64_t ca = N / 256; ca >= 0; --ca) {
+      const int64_t split = ca * 256;
+      if (split >= N) continue;
+      const double t = mixed_makespan(tm * ca, tm * ceil_div(N - split, 192), narrow_cost, cus);
+      if (t < best - 1e-6) best = t, best_split = split;
+    }
+  }
+  memo[memo_next] = Memo{M, N, cus, best_split};
+  memo_next = (memo_next + 1) % 8;
+  return best_split;
+}
+
 struct Plan {
   int variant;
   int bm, bn;
@@ -246,6 +291,7 @@ void tile_dims(int variant, int* bm, int* bn) {
       *bm = 128, *bn = 256;
       break;
     case kVarPipe256x256:
+    case kVarPipe256mix:
       *bm = 256, *bn = 256;
       break;
     default:
@@ -255,7 +301,7 @@ void tile_dims(int variant, int* bm, int* bn) {
 
 bool is_skinny(int v) { return v >= kVarSkinny16 && v <= kVarSkinny128; }
 int skinny_rows(int v) { return 16 << (v - kVarSkinny16); }
-bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe128x256w8; }
+bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe256mix; }
 
 // Largest split count (<= limit) whose slices still hold `min_kb` K blocks each.
 int pick_splitk(int64_t units, int kblocks, int cus, int waves_per_unit, int min_kb, int limit) {
@@ -282,7 +328,7 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
     } else if (whole_blocks && mode == kDense) {
       const int64_t t256 = ceil_div(M, 256) * ceil_div(N, 256);
       const int64_t t128 = ceil_div(M, 128) * ceil_div(N, 256);
-      v = t256 * 2 >= cus ? kVarPipe256x256 : (t128 * 4 >= cus ? kVarPipe128x256w8 : kVarTile128x128);
+      v = t256 * 2 >= cus ? kVarPipe256mix : (t128 * 4 >= cus ? kVarPipe128x256w8 : kVarTile128x128);
     } else if (whole_blocks) {
       v = kVarPipe128x256w8;  // grouped: 128-row tiles never straddle two experts / waste at most 127 masked rows
     } else {
@@ -292,7 +338,8 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
   if (K % 16 != 0) v = kVarExact;
   if (is_pipelined(v) && (K % kScaleBlock != 0 || K == 0)) v = kVarTile128x128;  // DMA path moves whole K blocks
   if (v == kVarPipe256x128 && mode == kContiguous) v = kVarPipe128x256;       // a tile must not straddle experts
-  if (v == kVarPipe256x256 && mode == kContiguous) v = kVarPipe128x256w8;
+  if ((v == kVarPipe256x256 || v == kVarPipe256mix) && mode == kContiguous) v = kVarPipe128x256w8;
+  if (v == kVarPipe256mix && mode != kDense) v = kVarPipe256x256;
   if (is_skinny(v) && (mode != kDense || M > skinny_rows(v))) v = kVarTile128x128;
   if (v == kVarExact && mode != kDense) v = kVarTile128x128;
   pl.variant = v;
@@ -477,7 +524,25 @@ int run(const Problem& pr) {
       }
       if (grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)grid);
       const int g = static_cast<int>(grid);
-      if (pl.variant == kVarPipe256x128)
+      if (pl.variant == kVarPipe256mix) {
+        const int64_t split = pick_mixed_split(pr.rows, pr.N, cus);
+        if (split >= pr.N) {
+          e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g, dev, pr.stream);
+        } else {
+          static std::atomic<unsigned long long> lds_done{0};
+          auto kernel = fp8_gemm_pipelined_mixed_kernel<Pipe256x256, Pipe256x192>;
+          ar.n_split = static_cast<int>(split);
+          ar.tiles_n_a = static_cast<int>(split / 256);
+          ar.tiles_n_b = static_cast<int>(ceil_div(pr.N - split, 192));
+          ar.tiles_a = ar.tiles_m * ar.tiles_n_a;
+          e = ensure_lds(kernel, Pipe256x256::LDS_BYTES, dev, &lds_done);
+          if (e == hipSuccess) {
+            hipLaunchKernelGGL(kernel, dim3(ar.tiles_a + ar.tiles_m * ar.tiles_n_b), dim3(Pipe256x256::NT),
+                               Pipe256x256::LDS_BYTES, pr.stream, ar);
+            e = hipGetLastError();
+          }
+        }
+      } else if (pl.variant == kVarPipe256x128)
         e = launch_pipelined_mode<Pipe256x128>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe128x256)
         e = launch_pipelined_mode<Pipe128x256>(pr.mode, ar, g, dev, pr.stream);

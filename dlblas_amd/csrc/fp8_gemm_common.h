@@ -52,6 +52,10 @@ struct Args {
   int group_m;          // m-tiles per L2 swizzle group
   int out_f32;
   int vec_store;        // rows of c are aligned for 4-element vector stores
+  int n_split;          // mixed-width launch: first column of the narrow-tile region
+  int tiles_a;          //   tiles in the wide region (tiles_m x tiles_n_a)
+  int tiles_n_a;
+  int tiles_n_b;
 };
 
 // D = A_op * B_op^T with A_op [16 x 128] and B_op [16 x 128] e4m3; lane l supplies row (l & 15) of each

@@ -88,6 +88,7 @@ template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_, int PARTS_ = 2, boo
 struct PipeCfg {
   static constexpr int WGM = WGM_, WGN = WGN_, MF = MF_, NF = NF_, STAGES = STAGES_, PARTS = PARTS_;
   static constexpr bool PREFETCH = PREFETCH_;
+  static constexpr bool UNIFORM_W = (128 % (NF_ * 32)) == 0;
   static constexpr int WAVES = WGM * WGN;
   static constexpr int NT = WAVES * 64;
   static constexpr int BM = WGM * MF * 32;
@@ -103,7 +104,7 @@ struct PipeCfg {
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
   static constexpr int LOADS_PER_STAGE = A_INST + B_INST + S_INST + 1;  // vmcnt units per wave and stage
   static_assert(BM % (8 * WAVES) == 0 && BN % (8 * WAVES) == 0, "tile rows must divide over the DMA instructions");
-  static_assert(NF * 32 <= 128 && 128 % (NF * 32) == 0, "a wave's n span must stay inside one 128-wide scale block");
+  static_assert(NF <= 4, "weight scales are fetched for at most four fragments per wave");
   static_assert(LOADS_PER_STAGE * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
 };
 
@@ -132,10 +133,16 @@ __global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* s
   }
 }
 
+// Work of one workgroup: tiles vb_first, vb_first + gridDim.x, ... of a region that is tiles_m x tiles_n tiles of
+// BM x BN and starts at column n_base of the output.
 template <class Cfg, int MODE>
-__global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args p) {
+__device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int vb_first, int tiles_m, int tiles_n,
+                                               int n_base) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MF = Cfg::MF, NF = Cfg::NF, WAVES = Cfg::WAVES, STAGES = Cfg::STAGES;
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // One weight scale per wave and K step when the wave's n span cannot straddle a 128-column scale block,
+  // otherwise one per 32-column fragment.
+  constexpr bool kUniformW = Cfg::UNIFORM_W;
+  constexpr int NS = kUniformW ? 1 : NF;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -146,18 +153,18 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
   const int wn0 = (wave % Cfg::WGN) * (NF * 32);
   const LaneChunks lc = make_lane_chunks(l32, h);
 
-  const int tiles = p.tiles_m * p.tiles_n;
+  const int tiles = tiles_m * tiles_n;
   int walk_g = 0;
   int walk_base = 0;
 
-  for (int vb = blockIdx.x;; vb += gridDim.x) {
+  for (int vb = vb_first;; vb += gridDim.x) {
     int g = 0, mt, nt, m_end;
     if (MODE == kMasked) {
       int mtiles = 0;
       while (walk_g < p.G) {
         const int valid = min(max(p.gidx[walk_g], 0), p.M);
         mtiles = (valid + BM - 1) / BM;
-        const int cnt = mtiles * p.tiles_n;
+        const int cnt = mtiles * tiles_n;
         if (vb < walk_base + cnt) break;
         walk_base += cnt;
         ++walk_g;
@@ -171,10 +178,10 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
     } else {
       if (vb >= tiles) break;
       const int t = xcd_remap(vb, tiles);
-      const int width = p.group_m * p.tiles_n;
+      const int width = p.group_m * tiles_n;
       const int grp = t / width;
       const int first_m = grp * p.group_m;
-      const int gsz = min(p.tiles_m - first_m, p.group_m);
+      const int gsz = min(tiles_m - first_m, p.group_m);
       const int in_grp = t - grp * width;
       mt = first_m + in_grp % gsz;
       nt = in_grp / gsz;
@@ -186,7 +193,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
     }
     g = __builtin_amdgcn_readfirstlane(g);
     const int m0 = __builtin_amdgcn_readfirstlane(mt * BM);
-    const int n0 = __builtin_amdgcn_readfirstlane(nt * BN);
+    const int n0 = __builtin_amdgcn_readfirstlane(n_base + nt * BN);
 
     const int64_t esz = p.out_f32 ? 4 : 2;
     const uint8_t* a_tile = p.a + static_cast<int64_t>(m0) * p.K;
@@ -198,8 +205,11 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
       c_base += static_cast<int64_t>(g) * p.c_gs * esz;
     }
     const uint8_t* b_tile = p.b + static_cast<int64_t>(g) * p.b_gs + static_cast<int64_t>(n0) * p.K;
-    const int nblk = __builtin_amdgcn_readfirstlane(min((n0 + wn0) / kScaleBlock, p.nblocks - 1));
-    const float* bs_row = p.b_s + static_cast<int64_t>(g) * p.bs_gs + static_cast<int64_t>(nblk) * p.kblocks;
+    // weight scales: lane i of the wave fetches the scale of the wave's fragment (i & 3) (fragment 0 beyond NF)
+    const float* bs_g = p.b_s + static_cast<int64_t>(g) * p.bs_gs;
+    const int bs_frag = (lane & 3) < NF ? (lane & 3) : 0;
+    const uint32_t bs_off =
+        static_cast<uint32_t>(min((n0 + wn0 + 32 * bs_frag) / kScaleBlock, p.nblocks - 1)) * static_cast<uint32_t>(p.kblocks) * 4u;
 
     // DMA addressing.  Instruction j of this wave fills LDS rows 8 (j WAVES + wave) .. + 7; lane i fills physical
     // chunk (i & 7) of row (i >> 3), which holds logical chunk (i & 7) ^ swizzle(row).  WAVES is even, so the
@@ -236,8 +246,8 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
         const uint32_t off = static_cast<uint32_t>(min(row, a_last)) * static_cast<uint32_t>(p.as_sm) * 4u;
         dma_4(sg, off, sbase + Cfg::A_BYTES + Cfg::B_BYTES + (j * WAVES + wave) * 256);
       }
-      // every lane of the wave fetches the same weight scale b_s[n block of this wave][kb] into its own LDS slot
-      dma_4(reinterpret_cast<const uint8_t*>(bs_row + kb), 0u,
+      // weight scales of the wave's fragments at this K block, one per lane slot
+      dma_4(reinterpret_cast<const uint8_t*>(bs_g + kb), bs_off,
             sbase + Cfg::A_BYTES + Cfg::B_BYTES + Cfg::S_BYTES + wave * 256);
     };
 
@@ -278,6 +288,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
     lds_barrier();
 
     if constexpr (Cfg::PREFETCH) {
+      static_assert(kUniformW, "the register-double-buffered path assumes one weight scale per wave");
       // ---- full register double buffering (one wave per SIMD) ------------------------------------------------
       v8i xr[2][MF][2];
       v8i wr[2][NF][2];
@@ -289,7 +300,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
       const int x0 = wm0 * kScaleBlock;
       const int w0 = (Cfg::BM + wn0) * kScaleBlock;
       auto load_scales = [&](int base, float (&dst)[MF]) {
-        const float sb = *reinterpret_cast<const float*>(smem + base + kWScaleOff + tid * 4);
+        const float sb = *reinterpret_cast<const float*>(smem + base + kWScaleOff + wave * 256);
         const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
 #pragma unroll
         for (int mi = 0; mi < MF; ++mi) dst[mi] = sS[wm0 + mi * 32 + l32] * sb;
@@ -363,17 +374,23 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
     } else {
     v8i hf[H][2];
     v8i sf[2];
-    float sc[MF];
+    float sc[MF][NS];
     float sc_last = 0.f;
     v16f part[2];
 #pragma unroll
     for (int u = 0; u < 16; ++u) part[0][u] = part[1][u] = 0.f;
 
-    auto load_scales = [&](int base, float (&dst)[MF]) {
-      const float sb = *reinterpret_cast<const float*>(smem + base + kWScaleOff + tid * 4);
+    auto load_scales = [&](int base, float (&dst)[MF][NS]) {
+      float sb[NS];
+#pragma unroll
+      for (int j = 0; j < NS; ++j) sb[j] = *reinterpret_cast<const float*>(smem + base + kWScaleOff + wave * 256 + j * 4);
       const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
 #pragma unroll
-      for (int mi = 0; mi < MF; ++mi) dst[mi] = sS[wm0 + mi * 32 + l32] * sb;
+      for (int mi = 0; mi < MF; ++mi) {
+        const float sa = sS[wm0 + mi * 32 + l32];
+#pragma unroll
+        for (int j = 0; j < NS; ++j) dst[mi][j] = sa * sb[j];
+      }
     };
     load_scales(0, sc);
 #pragma unroll
@@ -389,7 +406,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
       const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
       const int cur_base = stage * Cfg::STAGE_BYTES;
       const int nxt_base = next_stage * Cfg::STAGE_BYTES;
-      float sc_next[MF];
+      float sc_next[MF][NS];
 #pragma unroll
       for (int t = 0; t < T; ++t) {
         const int si = t / H, hi = t % H;
@@ -437,19 +454,21 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
         } else if (Cfg::PARTS == 1) {
           // scale-and-accumulate this tile; the other wave of the SIMD owns the matrix pipe meanwhile
           const int mi = kHoldX ? hi : si, ni = kHoldX ? si : hi;
-          acc[mi][ni] += part[0] * sc[mi];
+          acc[mi][ni] += part[0] * sc[mi][kUniformW ? 0 : ni];
         } else if (t == 0) {
           // scale-and-accumulate the previous tile while this tile's MFMAs run
           acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc_last;  // last tile of the previous K step (zero at kb = 0)
         } else {
           const int pt = t - 1;
           const int pmi = kHoldX ? pt % H : pt / H, pni = kHoldX ? pt / H : pt % H;
-          acc[pmi][pni] += part[pt & 1] * sc[pmi];
+          acc[pmi][pni] += part[pt & 1] * sc[pmi][kUniformW ? 0 : pni];
         }
       }
-      sc_last = sc[MF - 1];
+      sc_last = sc[MF - 1][NS - 1];
 #pragma unroll
-      for (int m2 = 0; m2 < MF; ++m2) sc[m2] = sc_next[m2];
+      for (int m2 = 0; m2 < MF; ++m2)
+#pragma unroll
+        for (int j = 0; j < NS; ++j) sc[m2][j] = sc_next[m2][j];
     };
     int stage = 0;
     for (int kb = 0; kb < nk; ++kb) {
@@ -480,6 +499,27 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
       }
     }
   }
+}
+
+template <class Cfg, int MODE>
+__global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  pipelined_body<Cfg, MODE>(p, smem, blockIdx.x, p.tiles_m, p.tiles_n, 0);
+}
+
+// Dense GEMM whose columns are cut at p.n_split into a region of CfgA tiles and a region of narrower CfgB tiles,
+// one workgroup per tile, region A first.  The host picks the cut so that the last round of workgroups fills the
+// chip: e.g. 448 tiles of 256 x 256 on 256 CUs leave a quarter of the chip idle in the second round, while 256
+// tiles of 256 x 256 followed by 256 tiles of 256 x 192 cover the same output and keep every CU busy.
+template <class CfgA, class CfgB>
+__global__ void __launch_bounds__(CfgA::NT) fp8_gemm_pipelined_mixed_kernel(const Args p) {
+  static_assert(CfgA::NT == CfgB::NT && CfgA::BM == CfgB::BM, "both regions use the same workgroup shape and tile height");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int bid = blockIdx.x;
+  if (bid < p.tiles_a)
+    pipelined_body<CfgA, kDense>(p, smem, bid, p.tiles_m, p.tiles_n_a, 0);
+  else
+    pipelined_body<CfgB, kDense>(p, smem, bid - p.tiles_a, p.tiles_m, p.tiles_n_b, p.n_split);
 }
 
 }  // namespace dlb

@@ -53,7 +53,7 @@ def test_dense_bf16_matches_oracle(dev, M, N, K):
     helpers.tolerance_check(out, ref, f'dense {M}x{N}x{K}')
 
 
-@pytest.mark.parametrize('variant', ['tile128x128', 'tile64x128', 'tile128x64', 'skinny16', 'skinny32', 'skinny64', 'skinny128', 'exact', 'pipe256x128', 'pipe128x256', 'pipe256x256', 'pipe128x256w8'])
+@pytest.mark.parametrize('variant', ['tile128x128', 'tile64x128', 'tile128x64', 'skinny16', 'skinny32', 'skinny64', 'skinny128', 'exact', 'pipe256x128', 'pipe128x256', 'pipe256x256', 'pipe128x256w8', 'pipe256mix'])
 @pytest.mark.parametrize('M,N,K', [(16, 512, 1024), (30, 200, 400), (200, 392, 2048)])
 def test_every_variant(dev, variant, M, N, K):
     print(f'case variant={variant} M={M} N={N} K={K}', flush=True)
