@@ -251,6 +251,19 @@ def grouped_workloads(dev):
     return rows
 
 
+def quantiser_workload(dev):
+    """The producer of (a, a_s): 1 x 128 quantisation of a bf16 [4096, 18432] activation; bytes = read + write."""
+    import torch
+
+    from dlblas_amd.kernels.fp8 import per_token_group_quant_fp8
+    M, K = 4096, 18432
+    x = torch.randn(M, K, device=dev, generator=torch.Generator(device=dev).manual_seed(20)).to(torch.bfloat16)
+    ms = time_call(lambda: per_token_group_quant_fp8(x, 128), 30, 5)
+    nbytes = 2 * M * K + M * K + 4 * M * (K // 128)
+    return {'workload': f'quant_1x128_bf16_{M}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
+            'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes}
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 --pmc runs kept under profiles/ (None when
     no counter run for this workload has been recorded)."""
@@ -337,6 +350,7 @@ def main():
                             'note': '24 distinct weight copies in rotation (353 MB) so reads miss the 256 MB cache'}
         log('grouped workloads')
         others += grouped_workloads(dev)
+        others.append(quantiser_workload(dev))
         result['other_workloads'] = others
 
     if args.copy_calibration:

@@ -32,6 +32,7 @@ SYMBOLS = {
     (ctypes.c_int, [_c_vp] * 6 + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 2 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_grouped_masked':
     (ctypes.c_int, [_c_vp] * 6 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 3 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
+    'dlb_fp8_quant_1x128': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
     'dlb_fp8_gemm_tune': (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
@@ -184,3 +185,16 @@ def gemm_masked(a, b, a_s, b_s, c, masked_m, expected_m, M_max, N, K, G, as_sg, 
             lib.dlb_fp8_gemm_grouped_masked(_ptr(a), _ptr(b), _ptr(a_s), _ptr(b_s), _ptr(c), _ptr(masked_m),
                                             int(expected_m), M_max, N, K, G, as_sg, as_sm, as_sk,
                                             out_code(c.dtype), _ptr(ws), ws.numel(), ctypes.c_void_p(stream)))
+
+
+IN_CODES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+
+def quant_1x128(x2d, q, s, rows, K, x_row_stride, s_stride_m, s_stride_k, eps):
+    _require_gpu(x2d, q, s)
+    lib = load()
+    with torch.cuda.device(x2d.device):
+        stream = torch.cuda.current_stream(x2d.device).cuda_stream
+        check(
+            lib.dlb_fp8_quant_1x128(_ptr(x2d), IN_CODES[x2d.dtype], _ptr(q), _ptr(s), rows, K, x_row_stride, s_stride_m,
+                                    s_stride_k, float(eps), ctypes.c_void_p(stream)))

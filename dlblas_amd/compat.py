@@ -13,6 +13,7 @@ _ALIASES = {
     'dlblas': 'dlblas_amd',
     'dlblas.kernels': 'dlblas_amd.kernels',
     'dlblas.kernels.fp8_gemm': 'dlblas_amd.kernels.fp8_gemm',
+    'dlblas.kernels.fp8': 'dlblas_amd.kernels.fp8',
     'dlblas.utils': 'dlblas_amd.utils',
     'dlblas.utils.logger': 'dlblas_amd.utils.logger',
     'dlblas.op_registry': 'dlblas_amd.op_registry',

@@ -14,6 +14,7 @@
 #include "fp8_gemm_pipelined.h"
 #include "fp8_gemm_skinny.h"
 #include "fp8_gemm_tiled.h"
+#include "fp8_quant.h"
 
 namespace dlb {
 
@@ -611,6 +612,40 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
   dlb::Problem pr{dlb::kMasked, a, b, a_s, b_s, c, masked_m, M_max, N, K, G, as_stride_g, as_stride_m, as_stride_k,
                   out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
   return dlb::run(pr);
+}
+
+int dlb_fp8_quant_1x128(const void* x, int x_dtype, void* q, float* s, int64_t rows, int64_t K, int64_t x_row_stride,
+                        int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream) {
+  using namespace dlb;
+  g_err[0] = '\0';
+  if (x_dtype < kInBf16 || x_dtype > kInF32) return fail(DLB_ERR_BAD_DTYPE, "x_dtype %d is not DLB_IN_BF16 / F16 / F32", x_dtype);
+  if (rows < 0 || K < 0) return fail(DLB_ERR_BAD_SHAPE, "negative dimension (rows=%lld K=%lld)", (long long)rows, (long long)K);
+  if (K % kScaleBlock != 0) return fail(DLB_ERR_BAD_SHAPE, "K=%lld is not a multiple of the group size 128", (long long)K);
+  if (rows == 0 || K == 0) return DLB_OK;
+  if (!x || !q || !s) return fail(DLB_ERR_NULL_POINTER, "x, q or s is NULL");
+  const int64_t esz = x_dtype == kInF32 ? 4 : 2;
+  if (x_row_stride < K) return fail(DLB_ERR_BAD_STRIDE, "x row stride %lld < K", (long long)x_row_stride);
+  if (s_stride_m < 0 || s_stride_k < 0) return fail(DLB_ERR_BAD_STRIDE, "negative scale stride");
+  if (misaligned(x, 16) || (x_row_stride * esz) % 16 != 0 || misaligned(q, 8) || misaligned(s, 4))
+    return fail(DLB_ERR_ALIGNMENT, "x rows must be 16-byte aligned, q 8-byte aligned");
+  int dev = 0;
+  const int cus = device_cu_count(&dev);
+  if (cus < 0) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
+  QuantArgs qa{x, static_cast<uint8_t*>(q), s, rows, K / kScaleBlock, x_row_stride, s_stride_m, s_stride_k, eps};
+  const int64_t groups = rows * (K / kScaleBlock);
+  int64_t blocks = ceil_div(groups, 16);  // 4 waves x 4 groups per step
+  const int64_t cap = static_cast<int64_t>(cus) * 16;
+  if (blocks > cap) blocks = cap;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (x_dtype == kInBf16)
+    hipLaunchKernelGGL(fp8_quant_1x128_kernel<kInBf16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, qa);
+  else if (x_dtype == kInF16)
+    hipLaunchKernelGGL(fp8_quant_1x128_kernel<kInF16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, qa);
+  else
+    hipLaunchKernelGGL(fp8_quant_1x128_kernel<kInF32>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, qa);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return DLB_OK;
 }
 
 int dlb_fp8_gemm_force_variant(int variant) {

@@ -1,0 +1,88 @@
+// 1 x 128 activation quantiser for gfx950: per row and 128-wide group, s = max(amax, eps) / 448 and
+// q = clamp(x / s, -448, 448) rounded to nearest-even e4m3fn.  Restates _per_token_group_quant_fp8 and its
+// column-major-scale twin (dlblas/kernels/fp8.py:8-105).  HBM-bound: every element is read once (16-byte loads,
+// 8 elements per lane) and written once (8-byte stores); 16 lanes share a group and reduce its amax with DPP-style
+// shuffles, so a wave handles 4 groups per step.
+#pragma once
+
+#include "fp8_gemm_common.h"
+
+namespace dlb {
+
+struct QuantArgs {
+  const void* x;
+  uint8_t* q;
+  float* s;
+  int64_t rows;
+  int64_t groups_per_row;  // K / 128
+  int64_t x_row_stride;    // elements
+  int64_t s_stride_m;      // floats
+  int64_t s_stride_k;
+  float eps;
+};
+
+enum QuantIn : int { kInBf16 = 0, kInF16 = 1, kInF32 = 2 };
+
+template <int IN>
+__device__ __forceinline__ void quant_load8(const void* x, int64_t elem, float (&v)[8]) {
+  if (IN == kInF32) {
+    const v4f* p = reinterpret_cast<const v4f*>(static_cast<const float*>(x) + elem);
+    const v4f a = p[0], b = p[1];
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+  } else {
+    const v4i raw = *reinterpret_cast<const v4i*>(static_cast<const uint16_t*>(x) + elem);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t w = static_cast<uint32_t>(raw[i]);
+      if (IN == kInBf16) {
+        v[2 * i] = __uint_as_float(w << 16);
+        v[2 * i + 1] = __uint_as_float(w & 0xffff0000u);
+      } else {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 hv = __builtin_bit_cast(h2, w);
+        v[2 * i] = static_cast<float>(hv.x);
+        v[2 * i + 1] = static_cast<float>(hv.y);
+      }
+    }
+  }
+}
+
+template <int IN>
+__global__ void __launch_bounds__(256) fp8_quant_1x128_kernel(const QuantArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int sub = lane & 15;  // position inside the group: elements 8 sub .. 8 sub + 7
+  const int64_t total = p.rows * p.groups_per_row;
+  const int64_t wave_id = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) >> 6;
+  const int64_t n_waves = (static_cast<int64_t>(gridDim.x) * 256) >> 6;
+  for (int64_t g0 = wave_id * 4; g0 < total; g0 += n_waves * 4) {
+    const int64_t g = g0 + (lane >> 4);
+    const bool live = g < total;
+    const int64_t gc = live ? g : total - 1;
+    const int64_t row = gc / p.groups_per_row;
+    const int64_t kg = gc - row * p.groups_per_row;
+    float v[8];
+    quant_load8<IN>(p.x, row * p.x_row_stride + kg * 128 + sub * 8, v);
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 16));
+    const float scale = fmaxf(amax, p.eps) / 448.0f;
+    int packed[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      float c[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) c[j] = fminf(fmaxf(v[4 * i + j] / scale, -448.0f), 448.0f);
+      int w = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], w, true);
+      packed[i] = w;
+    }
+    if (live) {
+      *reinterpret_cast<v2i*>(p.q + (row * p.groups_per_row + kg) * 128 + sub * 8) = v2i{packed[0], packed[1]};
+      if (sub == 0) p.s[row * p.s_stride_m + kg * p.s_stride_k] = scale;
+    }
+  }
+}
+
+}  // namespace dlb

@@ -1,0 +1,86 @@
+"""Activation quantiser that produces the (a, a_s) operands of the FP8 block-scaled GEMM.
+
+Drop-in for ``per_token_group_quant_fp8`` of the reference (dlblas/kernels/fp8.py:108-182): same signature, same
+assertions, same output shapes (including the column-major scale view), computed by a hand-written gfx950 kernel
+through the C ABI.  Only group_size 128 and float8_e4m3fn are implemented (the block-scaled GEMM takes nothing else).
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _lib
+from ..utils import SymVar, Tensor, register_dlblas_op
+
+
+@torch.library.custom_op('dlblas::per_token_group_quant_fp8', mutates_args=('x_q', 'x_s'), device_types='cuda')
+def quant_op(x: torch.Tensor, x_q: torch.Tensor, x_s: torch.Tensor, eps: float) -> None:
+    K = x.shape[-1]
+    rows = x.numel() // K
+    row_stride = x.stride(-2) if x.dim() >= 2 else K
+    _lib.quant_1x128(x, x_q, x_s, rows, K, row_stride, x_s.stride(-2) if x_s.dim() >= 2 else K // 128, x_s.stride(-1), eps)
+
+
+def per_token_group_quant_fp8(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    dtype: Optional[torch.dtype] = torch.float8_e4m3fn,
+    column_major_scales: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-token-group quantisation of ``x`` [..., K] (ndim >= 2, last dim contiguous) to float8_e4m3fn.
+
+    Returns ``(x_q, x_s)``: ``x_q`` like ``x`` in fp8, ``x_s`` fp32 ``[..., K / group_size]`` (a column-major view
+    when ``column_major_scales``), with ``x_s = max(amax, eps) / 448`` per group.
+    """
+    assert (x.shape[-1] % group_size == 0), (
+        f"the last dimension of 'x' {x.shape[-1]} must be divisible by 'group_size' {group_size}")
+    assert x.stride(-1) == 1, f'{x} groups must be contiguous'
+    if group_size != 128:
+        raise NotImplementedError(f'only group_size 128 is implemented, got {group_size}')
+    if dtype != torch.float8_e4m3fn:
+        raise NotImplementedError(f'only float8_e4m3fn is implemented, got {dtype}')
+    if x.dtype not in _lib.IN_CODES:
+        raise TypeError(f'x must be bfloat16, float16 or float32, got {x.dtype}')
+    if x.dim() < 2:
+        raise ValueError('x must have at least two dimensions')
+    K = x.shape[-1]
+    if x.dim() > 2 and not x.is_contiguous():
+        x = x.contiguous()
+    x2d = x if x.dim() == 2 else x.reshape(-1, K)
+    rows = x2d.shape[0]
+    x_q = torch.empty(x.shape, device=x.device, dtype=dtype)
+    if column_major_scales:
+        # the reference's layout: a [K / group, rows...] buffer viewed with the group axis last
+        buf = torch.empty((K // group_size, rows), device=x.device, dtype=torch.float32)
+        s2d = buf.t()
+        x_s = s2d if x.dim() == 2 else buf.reshape((K // group_size, ) + x.shape[:-1]).movedim(0, -1)
+    else:
+        x_s = torch.empty(x.shape[:-1] + (K // group_size, ), device=x.device, dtype=torch.float32)
+        s2d = x_s.reshape(rows, K // group_size)
+    quant_op(x2d, x_q.reshape(-1, K), s2d, float(eps))
+    return x_q, x_s
+
+
+def _bench(x, group_size, warmup: int = 3, rep: int = 10) -> float:
+    for _ in range(warmup):
+        per_token_group_quant_fp8(x, group_size)
+    times = []
+    for _ in range(rep):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        per_token_group_quant_fp8(x, group_size)
+        stop.record()
+        stop.synchronize()
+        times.append(start.elapsed_time(stop))
+    times.sort()
+    return times[len(times) // 2]
+
+
+def _register():
+    m, k = SymVar('m'), SymVar('k')
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        register_dlblas_op('per_token_group_quant_fp8', None, (Tensor((m, k), dtype=dt, device='cuda'), torch.SymInt),
+                           per_token_group_quant_fp8, _bench, per_token_group_quant_fp8)
+
+
+_register()

@@ -141,6 +141,26 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
                                 int64_t as_stride_g, int64_t as_stride_m, int64_t as_stride_k,
                                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* element type of the quantiser input */
+#define DLB_IN_BF16 0
+#define DLB_IN_F16 1
+#define DLB_IN_F32 2
+
+/*
+ * 1 x 128 activation quantiser, the producer of (a, a_s).  Replaces _per_token_group_quant_fp8 and
+ * _per_token_group_quant_fp8_colmajor behind per_token_group_quant_fp8 (dlblas/kernels/fp8.py:8-182) for
+ * group_size 128 and dtype float8_e4m3fn:
+ *     s[m, g] = max(max_k |x[m, 128 g + k]|, eps) / 448,   q = round_to_nearest_even_e4m3(clamp(x / s, -448, 448))
+ *
+ *   x  [rows, K]      bf16 / fp16 / fp32 (x_dtype), K contiguous, row stride x_row_stride elements, rows 16-byte aligned
+ *   q  [rows, K]      e4m3fn, contiguous
+ *   s  [rows, K/128]  fp32, element (m, g) at s[m * s_stride_m + g * s_stride_k]  (row- or column-major)
+ *
+ * K % 128 == 0 is required (the reference asserts divisibility by the group size).
+ */
+int dlb_fp8_quant_1x128(const void* x, int x_dtype, void* q, float* s, int64_t rows, int64_t K, int64_t x_row_stride,
+                        int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream);
+
 /*
  * Tuning / test hook: force the kernel variant the next calls FROM THIS THREAD use.
  * variant < 0 restores the built-in shape heuristic.  Returns DLB_ERR_BAD_SHAPE for an unknown id.

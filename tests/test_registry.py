@@ -20,7 +20,7 @@ def _cpu_args(dtype=torch.float32):
 
 def test_fp8_ops_are_registered_at_import():
     names = get_list_op_names()
-    for name in ('fp8_gemm', 'fp8_gemm_grouped_contiguous', 'fp8_gemm_grouped_masked'):
+    for name in ('fp8_gemm', 'fp8_gemm_grouped_contiguous', 'fp8_gemm_grouped_masked', 'per_token_group_quant_fp8'):
         assert name in names
     (params, ) = get_args_from_op_name('fp8_gemm')
     assert params.n_args == 4 and params.args_types == ['tensor'] * 4
