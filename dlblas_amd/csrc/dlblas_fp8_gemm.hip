@@ -51,8 +51,16 @@ namespace {
 
 thread_local char g_err[256] = "";
 thread_local int g_forced_variant = -1;
-enum Knob : int { kKnobSplitK = 0, kKnobSkinnyWaves, kKnobSkinnyUnroll, kKnobSkinnyNFrags, kKnobGroupM, kKnobCount };
-thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0};
+enum Knob : int {
+  kKnobSplitK = 0,
+  kKnobSkinnyWaves,
+  kKnobSkinnyUnroll,
+  kKnobSkinnyNFrags,
+  kKnobGroupM,
+  kKnobSkinnyDma,  // 0 / 1: DMA-staged decode kernel where possible, 2: register-load decode kernel
+  kKnobCount
+};
+thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0};
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -166,8 +174,16 @@ hipError_t launch_pipelined_mode(int mode, const Args& args, int grid, int dev, 
 
 template <class Cfg>
 hipError_t launch_skinny_cfg(const Args& args, int dev, hipStream_t stream) {
-  static std::atomic<unsigned long long> lds_done{0}, lds_done_tail{0};
+  static std::atomic<unsigned long long> lds_done{0}, lds_done_tail{0}, lds_done_dma{0};
   const bool ktail = args.K % kScaleBlock != 0;
+  // full-line DMA staging where it fits in LDS and K has no ragged block; else the register-load kernel
+  if (!ktail && Cfg::DMA_LDS_BYTES <= 160 * 1024 && g_knob[kKnobSkinnyDma] != 2) {
+    auto kernel = fp8_gemm_skinny_dma_kernel<Cfg>;
+    hipError_t e = ensure_lds(kernel, Cfg::DMA_LDS_BYTES, dev, &lds_done_dma);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3(args.tiles_n), dim3(Cfg::NT), Cfg::DMA_LDS_BYTES, stream, args);
+    return hipGetLastError();
+  }
   auto kernel = ktail ? fp8_gemm_skinny_kernel<Cfg, true> : fp8_gemm_skinny_kernel<Cfg, false>;
   hipError_t e = ensure_lds(kernel, Cfg::RED_BYTES, dev, ktail ? &lds_done_tail : &lds_done);
   if (e != hipSuccess) return e;

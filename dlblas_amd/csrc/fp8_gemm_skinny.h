@@ -23,6 +23,7 @@ struct SkinnyCfg {
   static constexpr int NT = WAVES * 64;
   static constexpr int BN = 16 * NFS;
   static constexpr int RED_BYTES = WAVES * MF * NFS * 64 * 16;
+  static constexpr int DMA_LDS_BYTES = WAVES * UNROLL * (NFS + MF) * 2048 + RED_BYTES;  // staging + reduction
 };
 
 // 32 operand bytes of one lane for K block `kb`: bytes [16 q, 16 q + 16) and [64 + 16 q, 64 + 16 q + 16) of the
@@ -127,6 +128,153 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_kernel(const Args p) 
   __syncthreads();
 
   // fragment j of the output is summed (in wave order) and stored by wave j % WAVES
+  const int64_t esz = p.out_f32 ? 4 : 2;
+  for (int j = wave; j < MF * NFS; j += WAVES) {
+    const int mi = j / NFS, ni = j % NFS;
+    v4f sum = red[0][j][lane];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) sum += red[w][j][lane];
+    const int m = mi * 16 + l16;
+    const int n = n0 + ni * 16 + q * 4;
+    if (m >= p.M) continue;
+    char* c_row = static_cast<char*>(p.c) + static_cast<int64_t>(m) * p.N * esz;
+    if (p.out_f32)
+      store_row4<true>(c_row, n, sum, p.N - n, p.vec_store);
+    else
+      store_row4<false>(c_row, n, sum, p.N - n, p.vec_store);
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------------------------
+// Same computation with full-cache-line global accesses: every wave moves the 16 x 128-byte blocks of its K blocks
+// (weights AND activations) into a wave-private LDS area with the DMA path, 8 rows x 128 bytes per instruction, and
+// reads its MFMA operands back with ds_read_b128.  The register-load kernel above touches every line with two
+// half-line requests of 16 rows each; measured on MI355X that costs 1.3 us of a 7 us launch for the weights and
+// 2 us for the activations.  No barrier is involved: a wave only reads what it moved itself.  K % 128 == 0 only
+// (the DMA cannot zero-fill a ragged last block).
+// ---------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int skinny_swizzle(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args p) {
+  constexpr int MF = Cfg::MF, WAVES = Cfg::WAVES, U = Cfg::UNROLL, NFS = Cfg::NFS;
+  constexpr int FRAGS = NFS + MF;                 // 2 KB blocks per K block: weights first, then activations
+  constexpr int WAVE_BYTES = U * FRAGS * 2048;    // staging area of one wave
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  v4f(*red)[MF * NFS][64] = reinterpret_cast<v4f(*)[MF * NFS][64]>(smem + WAVES * WAVE_BYTES);
+
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  typedef const __attribute__((address_space(1))) void* global_ptr_t;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15;
+  const int q = lane >> 4;
+  const int n0 = blockIdx.x * Cfg::BN;
+  const int nk = p.kblocks;
+  uint8_t* stage = smem + wave * WAVE_BYTES;
+
+  // DMA source offsets: instruction j (0 / 1) of a block fills rows 8 j .. 8 j + 7; lane i fills physical chunk
+  // (i & 7) of row 8 j + (i >> 3), which holds logical chunk (i & 7) ^ swizzle(row)
+  uint32_t w_off[NFS][2], x_off[MF][2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int row = 8 * j + (lane >> 3);
+    const uint32_t chunk = static_cast<uint32_t>(((lane & 7) ^ skinny_swizzle(row)) * 16);
+#pragma unroll
+    for (int ni = 0; ni < NFS; ++ni)
+      w_off[ni][j] = static_cast<uint32_t>(min(ni * 16 + row, p.N - 1 - n0)) * static_cast<uint32_t>(p.K) + chunk;
+#pragma unroll
+    for (int mi = 0; mi < MF; ++mi)
+      x_off[mi][j] = static_cast<uint32_t>(min(mi * 16 + row, p.M - 1)) * static_cast<uint32_t>(p.K) + chunk;
+  }
+  const uint8_t* w_base = p.b + static_cast<int64_t>(n0) * p.K;
+  // operand read offsets: lane (row = lane & 15, q) reads logical chunks 2 q and 2 q + 1 of its row
+  const int sw = skinny_swizzle(l16);
+  const int rd0 = l16 * 128 + (((2 * q) ^ sw) << 4);
+  const int rd1 = l16 * 128 + (((2 * q + 1) ^ sw) << 4);
+
+  const float* bs_row[NFS];
+#pragma unroll
+  for (int ni = 0; ni < NFS; ++ni)
+    bs_row[ni] = p.b_s + static_cast<int64_t>(min((n0 + ni * 16) / kScaleBlock, p.nblocks - 1)) * nk;
+  const float* as_row[MF];
+#pragma unroll
+  for (int mi = 0; mi < MF; ++mi) as_row[mi] = p.a_s + static_cast<int64_t>(min(mi * 16 + l16, p.M - 1)) * p.as_sm;
+
+  v4f acc[MF][NFS];
+#pragma unroll
+  for (int mi = 0; mi < MF; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NFS; ++ni) acc[mi][ni] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = wave; kb < nk; kb += WAVES * U) {
+    float sa[U][MF], sb[U][NFS];
+    // weights first: they are the HBM stream.  A K block past the end re-reads the last one with scale 0.
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kbu = min(kb + u * WAVES, nk - 1);
+      const uint8_t* wk = w_base + static_cast<int64_t>(kbu) * kScaleBlock;
+#pragma unroll
+      for (int ni = 0; ni < NFS; ++ni)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          __builtin_amdgcn_global_load_lds((global_ptr_t)(wk + w_off[ni][j]),
+                                           (lds_ptr_t)(stage + (u * FRAGS + ni) * 2048 + j * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool valid = kb + u * WAVES < nk;
+      const int kbu = min(kb + u * WAVES, nk - 1);
+      const uint8_t* xk = p.a + static_cast<int64_t>(kbu) * kScaleBlock;
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          __builtin_amdgcn_global_load_lds((global_ptr_t)(xk + x_off[mi][j]),
+                                           (lds_ptr_t)(stage + (u * FRAGS + NFS + mi) * 2048 + j * 1024), 16, 0, 0);
+#pragma unroll
+      for (int ni = 0; ni < NFS; ++ni) {
+        const float v = bs_row[ni][kbu];
+        sb[u][ni] = valid ? v : 0.f;
+      }
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) sa[u][mi] = as_row[mi][static_cast<int64_t>(kbu) * p.as_sk];
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): this wave's DMA groups have landed in its LDS area
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      v8i wf[NFS], xf[MF];
+#pragma unroll
+      for (int f = 0; f < FRAGS; ++f) {
+        const uint8_t* blk = stage + (u * FRAGS + f) * 2048;
+        const v4i lo = *reinterpret_cast<const v4i*>(blk + rd0);
+        const v4i hi = *reinterpret_cast<const v4i*>(blk + rd1);
+        const v8i v = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        if (f < NFS)
+          wf[f] = v;
+        else
+          xf[f - NFS] = v;
+      }
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NFS; ++ni) {
+          const v4f part = mfma_16x16x128_e4m3(wf[ni], xf[mi], v4f{0.f, 0.f, 0.f, 0.f});
+          acc[mi][ni] += part * (sa[u][mi] * sb[u][ni]);
+        }
+    }
+    // the next round of DMA overwrites the staging area: its reads above have returned (their values were used)
+  }
+
+#pragma unroll
+  for (int mi = 0; mi < MF; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < NFS; ++ni) red[wave][mi * NFS + ni][lane] = acc[mi][ni];
+  __syncthreads();
+
   const int64_t esz = p.out_f32 ? 4 : 2;
   for (int j = wave; j < MF * NFS; j += WAVES) {
     const int mi = j / NFS, ni = j % NFS;

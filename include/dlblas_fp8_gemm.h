@@ -175,12 +175,14 @@ int dlb_fp8_gemm_force_variant(int variant);
  *   DLB_KNOB_SKINNY_UNROLL  K blocks a decode-kernel wave loads before its first MFMA (1, 2 or 4)
  *   DLB_KNOB_SKINNY_NFRAGS  16-row weight fragments per decode workgroup (1 or 2)
  *   DLB_KNOB_GROUP_M        m-tiles per L2 swizzle group of the tiled kernels
+ *   DLB_KNOB_SKINNY_DMA     2 = decode kernels load operands through registers instead of the LDS DMA path
  */
 #define DLB_KNOB_SPLITK 0
 #define DLB_KNOB_SKINNY_WAVES 1
 #define DLB_KNOB_SKINNY_UNROLL 2
 #define DLB_KNOB_SKINNY_NFRAGS 3
 #define DLB_KNOB_GROUP_M 4
+#define DLB_KNOB_SKINNY_DMA 5
 int dlb_fp8_gemm_tune(int knob, int value);
 
 /* Name of kernel variant `variant`, or NULL beyond the last one. */
