@@ -30,8 +30,8 @@ struct Args {
   const float* b_s;
   void* c;
   const int32_t* gidx;  // m_indices (contiguous) / masked_m (masked) / nullptr (dense)
-  float* ws;            // split-K partial tiles
-  uint32_t* ctr;        // split-K arrival counters, one per output tile, zero between calls
+  float* ws;            // scratch: split-K partial matrices [splitk][M][N]
+  uint32_t* ctr;        // reserved head of the workspace (unused)
   int64_t a_gs;         // per-expert strides in elements (masked mode)
   int64_t as_gs;
   int64_t c_gs;

@@ -70,7 +70,6 @@ template <class Cfg, int MODE>
 __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_tiled_kernel(const Args p) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, NT = Cfg::NT, MF = Cfg::MF, NF = Cfg::NF;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  __shared__ int s_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -214,37 +213,23 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_tiled_kernel(const Args p) {
     }
 
     if (MODE == kDense && p.splitk > 1) {
-      // Deterministic split-K: every split parks its partial tile in the workspace; the workgroup that
-      // arrives last adds the splits in index order and runs the epilogue.
-      float* wst = p.ws + (static_cast<int64_t>(t) * p.splitk) * (BM * BN);
-      float* mine = wst + static_cast<int64_t>(split) * (BM * BN);
+      // Split-K, first pass: this workgroup's K slice goes to the workspace as a plain fp32 [M][N] matrix of its
+      // own; fp8_splitk_reduce_kernel, launched behind this kernel on the same stream, adds the slices in index
+      // order (deterministic) and casts.  No fence, no counter: stream order makes the partial sums visible.
+      float* mine = p.ws + static_cast<int64_t>(split) * p.M * p.N;
+      const bool vec_ok = (p.N % 4) == 0;
 #pragma unroll
-      for (int mi = 0; mi < MF; ++mi)
+      for (int mi = 0; mi < MF; ++mi) {
+        const int m = m0 + wm0 + mi * 16 + l16;
+        if (m >= m_end) continue;
+        float* w_row = mine + static_cast<int64_t>(m) * p.N;
 #pragma unroll
-        for (int ni = 0; ni < NF; ++ni)
-          *reinterpret_cast<v4f*>(mine + ((mi * NF + ni) * NT + tid) * 4) = acc[mi][ni];
-      __threadfence();
-      __syncthreads();
-      if (tid == 0) {
-        const unsigned prev = atomicAdd(&p.ctr[t], 1u);
-        s_last = (prev == static_cast<unsigned>(p.splitk - 1));
+        for (int ni = 0; ni < NF; ++ni) {
+          const int n = n0 + wn0 + ni * 16 + q * 4;
+          store_row4<true>(w_row, n, acc[mi][ni], p.N - n, vec_ok);
+        }
       }
-      __syncthreads();
-      if (!s_last) continue;
-      __threadfence();
-#pragma unroll
-      for (int mi = 0; mi < MF; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NF; ++ni) acc[mi][ni] = v4f{0.f, 0.f, 0.f, 0.f};
-      for (int s = 0; s < p.splitk; ++s) {
-        const float* src = wst + static_cast<int64_t>(s) * (BM * BN);
-#pragma unroll
-        for (int mi = 0; mi < MF; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < NF; ++ni)
-            acc[mi][ni] += __builtin_nontemporal_load(reinterpret_cast<const v4f*>(src + ((mi * NF + ni) * NT + tid) * 4));
-      }
-      if (tid == 0) p.ctr[t] = 0u;
+      continue;
     }
 
     // epilogue: lane holds c[m0 + wm0 + 16 mi + (lane & 15)][n0 + wn0 + 16 ni + 4 (lane >> 4) + 0..3]
@@ -263,6 +248,31 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_tiled_kernel(const Args p) {
       }
     }
   }
+}
+
+// Split-K, second pass: c[i] = sum over s (in index order) of ws[s][i], i over the M x N outputs, four per thread.
+__global__ void __launch_bounds__(256) fp8_splitk_reduce_kernel(const float* ws, void* c, int64_t total, int splits,
+                                                                int out_f32, int vec_ok) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  const int left = static_cast<int>(total - i < 4 ? total - i : 4);
+  v4f sum = {0.f, 0.f, 0.f, 0.f};
+  if (vec_ok) {  // total % 4 == 0 and 16-byte aligned slices
+    for (int s = 0; s < splits; ++s)
+      sum += __builtin_nontemporal_load(reinterpret_cast<const v4f*>(ws + static_cast<int64_t>(s) * total + i));
+  } else {
+    for (int s = 0; s < splits; ++s) {
+      const float* src = ws + static_cast<int64_t>(s) * total + i;
+      sum.x += src[0];
+      if (left > 1) sum.y += src[1];
+      if (left > 2) sum.z += src[2];
+      if (left > 3) sum.w += src[3];
+    }
+  }
+  if (out_f32)
+    store_row4<true>(c, i, sum, left, vec_ok != 0);
+  else
+    store_row4<false>(c, i, sum, left, vec_ok != 0);
 }
 
 }  // namespace dlb

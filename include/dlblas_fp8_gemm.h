@@ -17,10 +17,12 @@
  *     dlb_last_error() gives a thread-local human-readable reason for the last failure;
  *   - no C++ exception ever crosses this boundary;
  *   - `workspace` is caller-owned device memory of at least dlb_fp8_gemm_workspace_bytes()
- *     bytes.  Its first DLB_WS_COUNTER_BYTES bytes are tile counters: they must be ZERO the
- *     first time the buffer is used and are left zero by every call, so one buffer can be
- *     reused by any number of calls that do not overlap in time.  Two calls that may run
- *     concurrently (different streams) need separate workspaces.
+ *     bytes, 16-byte aligned.  Its first DLB_WS_COUNTER_BYTES bytes are reserved (no kernel
+ *     of this version reads or writes them); the rest is scratch that a call overwrites:
+ *     re-laid activation scales, fp32 partial sums of the split-K path.  Nothing in it has
+ *     to survive between calls, so one buffer serves any number of calls that do not overlap
+ *     in time.  Two calls that may run concurrently (different streams) need separate
+ *     workspaces.
  *
  * Reference interfaces these replace (paths relative to the DLBlas source tree):
  *   - dlb_fp8_gemm                     : dlblas/kernels/fp8_gemm.py:15-65 (kernel) and :68-89 (host wrapper)
@@ -58,7 +60,7 @@ extern "C" {
 #define DLB_ERR_ALIGNMENT (-6)      /* a pointer is not 16-byte aligned where the kernels need it  */
 #define DLB_ERR_LAUNCH (-7)         /* the HIP runtime refused the launch                          */
 
-/* bytes at the head of every workspace that hold self-resetting tile counters */
+/* reserved bytes at the head of every workspace */
 #define DLB_WS_COUNTER_BYTES 65536
 
 /* Version of this ABI (DLB_ABI_VERSION of the library that was loaded). */
@@ -170,7 +172,8 @@ int dlb_fp8_gemm_force_variant(int variant);
 
 /*
  * Tuning / test hook: set knob `knob` for the next calls FROM THIS THREAD; value 0 restores the heuristic.
- *   DLB_KNOB_SPLITK         K splits of the LDS-tiled dense kernels (clamped to what workspace and K allow)
+ *   DLB_KNOB_SPLITK         K slices of the LDS-tiled dense kernels, each summed into its own fp32 matrix in the workspace and added
+ *                           by a second kernel in slice order (clamped to what workspace and K allow)
  *   DLB_KNOB_SKINNY_WAVES   waves per workgroup of the decode kernels (4, 8 or 16)
  *   DLB_KNOB_SKINNY_UNROLL  K blocks a decode-kernel wave loads before its first MFMA (1, 2 or 4)
  *   DLB_KNOB_SKINNY_NFRAGS  16-row weight fragments per decode workgroup (1 or 2)

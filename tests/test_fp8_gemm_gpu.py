@@ -63,6 +63,27 @@ def test_every_variant(dev, variant, M, N, K):
     helpers.tolerance_check(out, ref, f'{variant} {M}x{N}x{K}')
 
 
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('variant,splitk', [('tile128x128', 2), ('tile128x64', 5), ('tile64x128', 32), (None, 0)])
+@pytest.mark.parametrize('M,N,K', [(128, 2112, 7168), (200, 392, 2048), (129, 130, 1040), (70, 131, 4096)])
+def test_split_k_two_pass(dev, M, N, K, variant, splitk, out_dtype):
+    """K split over workgroups: fp32 partial matrices in the workspace, a second kernel adds them in index order.
+    (None, 0) is the library's own choice, which splits (128, 2112, 7168).  Two calls must agree bit for bit."""
+    from dlblas_amd import _lib
+    print(f'case split-K variant={variant} splitk={splitk} M={M} N={N} K={K} {out_dtype}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=11)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    try:
+        _lib.force_splitk(splitk)
+        out = _run_dense(dev, a_q, a_s, b_q, b_s, dtype=out_dtype, variant=variant)
+        again = _run_dense(dev, a_q, a_s, b_q, b_s, dtype=out_dtype, variant=variant)
+    finally:
+        _lib.force_splitk(0)
+    assert out.dtype == out_dtype
+    helpers.tolerance_check(out, ref, f'split-K {variant}/{splitk} {M}x{N}x{K}')
+    assert torch.equal(out, again)
+
+
 def test_dense_f32_reference_test_construction(dev):
     """The reference's own test: randn e4m3 operands, randn (signed) scales, fp32 out, atol 1e-1
     (tests/kernels/test_fp8_gemm.py:8-31,70-72)."""
