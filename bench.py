@@ -258,10 +258,57 @@ def quantiser_workload(dev):
     from dlblas_amd.kernels.fp8 import per_token_group_quant_fp8
     M, K = 4096, 18432
     x = torch.randn(M, K, device=dev, generator=torch.Generator(device=dev).manual_seed(20)).to(torch.bfloat16)
-    ms = time_call(lambda: per_token_group_quant_fp8(x, 128), 30, 5)
+    from dlblas_amd import _lib
+    x_q, x_s = per_token_group_quant_fp8(x, 128)
+    lib = _lib.load()
+    vp = ctypes.c_void_p
+    args = (vp(x.data_ptr()), _lib.IN_CODES[x.dtype], vp(x_q.data_ptr()), vp(x_s.data_ptr()), M, K, K, K // 128, 1, 1e-10,
+            vp(torch.cuda.current_stream().cuda_stream))
+    ms = time_call(lambda: lib.dlb_fp8_quant_1x128(*args), 100, 10)
     nbytes = 2 * M * K + M * K + 4 * M * (K // 128)
     return {'workload': f'quant_1x128_bf16_{M}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
             'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes}
+
+
+def activation_workloads(dev):
+    """The step between the two grouped GEMMs: silu(gate) * up + 1 x 128 quantisation.  Contiguous layout at the
+    expert-contiguous shape (9728 padded rows, gate_up 4096 wide -> 2048 fp8), masked layout at the decode shape
+    (32 experts x 256 rows capacity, gate_up 4096 wide).  bytes = bf16 read + fp8 and scale written (valid rows)."""
+    import torch
+
+    from dlblas_amd import _lib
+    gd = torch.Generator(device=dev).manual_seed(20)
+    rows = []
+    M, N = 9728, 2048
+    x = torch.randn(M, 2 * N, device=dev, generator=gd).to(torch.bfloat16)
+    q2 = torch.empty(M, N, device=dev, dtype=torch.float8_e4m3fn)
+    s2 = torch.empty(M, N // 128, device=dev, dtype=torch.float32)
+    # pre-marshalled C calls with caller-owned outputs: the kernels take 10-30 us, less than a torch op dispatch
+    lib = _lib.load()
+    vp = ctypes.c_void_p
+    stream = vp(torch.cuda.current_stream().cuda_stream)
+    args = (vp(x.data_ptr()), _lib.IN_CODES[x.dtype], vp(q2.data_ptr()), vp(s2.data_ptr()), M, N, 2 * N, N // 128, 1, 1e-10, stream)
+    _lib.check(lib.dlb_silu_mul_quant(*args))
+    ms = time_call(lambda: lib.dlb_silu_mul_quant(*args), 100, 10)
+    nbytes = 4 * M * N + M * N + 4 * M * (N // 128)
+    rows.append({'workload': f'silu_mul_quant_bf16_{M}x{2 * N}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
+                 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes})
+    G, M_max = GROUPED_MASKED['G'], GROUPED_MASKED['M_max']
+    masked_m = torch.randint(0, M_max + 1, (G, ), generator=torch.Generator().manual_seed(20), dtype=torch.int32)
+    x3 = torch.randn(G, M_max, 2 * N, device=dev, generator=gd).to(torch.bfloat16)
+    q = torch.empty(G, M_max, N, device=dev, dtype=torch.float8_e4m3fn)
+    s = torch.empty(G, M_max, N // 128, device=dev, dtype=torch.float32)
+    mm = masked_m.to(dev)
+    args3 = (vp(x3.data_ptr()), _lib.IN_CODES[x3.dtype], vp(q.data_ptr()), vp(s.data_ptr()), vp(mm.data_ptr()), G, M_max, N,
+             s.stride(0), s.stride(1), s.stride(2), stream)
+    _lib.check(lib.dlb_silu_mul_quant_masked(*args3))
+    ms = time_call(lambda: lib.dlb_silu_mul_quant_masked(*args3), 100, 10)
+    valid = int(masked_m.sum())
+    nbytes = 4 * valid * N + valid * N + 4 * valid * (N // 128) + 4 * G
+    rows.append({'workload': f'silu_mul_quant_masked_bf16_E{G}_Mmax{M_max}_{2 * N}', 'valid_rows': valid,
+                 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                 'bytes': nbytes})
+    return rows
 
 
 def measured_traffic(workload):
@@ -351,6 +398,7 @@ def main():
         log('grouped workloads')
         others += grouped_workloads(dev)
         others.append(quantiser_workload(dev))
+        others += activation_workloads(dev)
         result['other_workloads'] = others
 
     if args.copy_calibration:

@@ -7,7 +7,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(PKG_DIR, 'csrc')
 LIB_NAME = 'libdlblas_fp8_gemm.so'
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = ['dlblas_fp8_gemm.hip']
+SOURCES = ['dlblas_fp8_gemm.hip', 'dlblas_fp8_moe.hip']
 
 # packed fp32 VALU forms are switched off for every device compile of this library
 HIPCC_FLAGS = [

@@ -1,4 +1,4 @@
-"""ctypes binding of libdlblas_fp8_gemm.so (the C ABI declared in include/dlblas_fp8_gemm.h).
+"""ctypes binding of libdlblas_fp8_gemm.so (the C ABI declared in include/dlblas_fp8_gemm.h and dlblas_fp8_moe.h).
 
 The library is the only implementation: when it has not been built, every op raises ImportError.  There is no
 PyTorch or CPU fallback.  The calling convention (``c_void_p(tensor.data_ptr())`` operands, the stream handle as
@@ -22,7 +22,7 @@ ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_BAD_STRIDE, ERR_BAD_DTYPE, ERR_WORKSPACE, E
 
 _c_i64, _c_i32, _c_vp, _c_sz = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.c_size_t
 
-# name -> (restype, argtypes); must list every symbol include/dlblas_fp8_gemm.h declares
+# name -> (restype, argtypes); must list every symbol the headers under include/ declare
 SYMBOLS = {
     'dlb_abi_version': (ctypes.c_int, []),
     'dlb_last_error': (ctypes.c_char_p, []),
@@ -36,6 +36,9 @@ SYMBOLS = {
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
     'dlb_fp8_gemm_tune': (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
+    'dlb_silu_mul': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp] + [_c_i64] * 4 + [_c_vp]),
+    'dlb_silu_mul_quant': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
+    'dlb_silu_mul_quant_masked': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp, _c_vp] + [_c_i64] * 6 + [_c_vp]),
 }
 
 _lock = threading.Lock()
@@ -198,3 +201,30 @@ def quant_1x128(x2d, q, s, rows, K, x_row_stride, s_stride_m, s_stride_k, eps):
         check(
             lib.dlb_fp8_quant_1x128(_ptr(x2d), IN_CODES[x2d.dtype], _ptr(q), _ptr(s), rows, K, x_row_stride, s_stride_m,
                                     s_stride_k, float(eps), ctypes.c_void_p(stream)))
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def silu_mul(x2d, out2d, rows, N):
+    lib = load()
+    _require_gpu(x2d, out2d)
+    with torch.cuda.device(x2d.device):
+        check(lib.dlb_silu_mul(_ptr(x2d), IN_CODES[x2d.dtype], _ptr(out2d), rows, N, x2d.stride(0), out2d.stride(0), _stream(x2d)))
+
+
+def silu_mul_quant(x2d, q, s, rows, N, s_stride_m, s_stride_k, eps):
+    lib = load()
+    _require_gpu(x2d, q, s)
+    with torch.cuda.device(x2d.device):
+        check(lib.dlb_silu_mul_quant(_ptr(x2d), IN_CODES[x2d.dtype], _ptr(q), _ptr(s), rows, N, x2d.stride(0), s_stride_m,
+                                     s_stride_k, float(eps), _stream(x2d)))
+
+
+def silu_mul_quant_masked(x, q, s, masked_m, G, M_max, N, s_strides):
+    lib = load()
+    _require_gpu(x, q, s, masked_m)
+    with torch.cuda.device(x.device):
+        check(lib.dlb_silu_mul_quant_masked(_ptr(x), IN_CODES[x.dtype], _ptr(q), _ptr(s), _ptr(masked_m), G, M_max, N,
+                                            s_strides[0], s_strides[1], s_strides[2], _stream(x)))

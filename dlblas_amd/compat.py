@@ -14,6 +14,8 @@ _ALIASES = {
     'dlblas.kernels': 'dlblas_amd.kernels',
     'dlblas.kernels.fp8_gemm': 'dlblas_amd.kernels.fp8_gemm',
     'dlblas.kernels.fp8': 'dlblas_amd.kernels.fp8',
+    'dlblas.kernels.moe': 'dlblas_amd.kernels.moe',
+    'dlblas.layers.moe.kernels.activation': 'dlblas_amd.kernels.activation',
     'dlblas.utils': 'dlblas_amd.utils',
     'dlblas.utils.logger': 'dlblas_amd.utils.logger',
     'dlblas.op_registry': 'dlblas_amd.op_registry',
@@ -34,8 +36,20 @@ def install(dlblas: bool = True, deep_gemm: bool = True) -> None:
     import importlib
     if dlblas:
         for alias, target in _ALIASES.items():
+            # intermediate packages this package has no counterpart for (dlblas.layers, dlblas.layers.moe, ...)
+            parts = alias.split('.')
+            for i in range(1, len(parts)):
+                parent = '.'.join(parts[:i])
+                if parent not in sys.modules and parent not in _ALIASES:
+                    pkg = types.ModuleType(parent)
+                    pkg.__path__ = []
+                    sys.modules[parent] = pkg
+                    if i > 1:
+                        setattr(sys.modules['.'.join(parts[:i - 1])], parts[i - 1], pkg)
             if alias not in sys.modules:
                 sys.modules[alias] = importlib.import_module(target)
+                if len(parts) > 1:
+                    setattr(sys.modules['.'.join(parts[:-1])], parts[-1], sys.modules[alias])
     if deep_gemm and 'deep_gemm' not in sys.modules:
         from .kernels import fp8_gemm_grouped as grouped
         mod = types.ModuleType('deep_gemm')

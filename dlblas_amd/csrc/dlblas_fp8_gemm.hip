@@ -11,6 +11,7 @@
 #include <cstring>
 
 #include "fp8_gemm_common.h"
+#include "host_common.h"
 #include "fp8_gemm_pipelined.h"
 #include "fp8_gemm_skinny.h"
 #include "fp8_gemm_tiled.h"
@@ -47,9 +48,35 @@ __global__ void __launch_bounds__(256) fp8_gemm_exact_kernel(const Args p) {
 // ---------------------------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------------------------
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void clear_error() { g_err[0] = '\0'; }
+
+int device_cu_count(int* dev_out) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  *dev_out = dev;
+  if (dev < 0 || dev >= kMaxDevices) return 256;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    cached[dev].store(cus, std::memory_order_relaxed);
+  }
+  return cus;
+}
+
 namespace {
 
-thread_local char g_err[256] = "";
 thread_local int g_forced_variant = -1;
 enum Knob : int {
   kKnobSplitK = 0,
@@ -61,14 +88,6 @@ enum Knob : int {
   kKnobCount
 };
 thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0};
-
-int fail(int code, const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_err, sizeof(g_err), fmt, ap);
-  va_end(ap);
-  return code;
-}
 
 enum Variant : int {
   kVarExact = 0,
@@ -99,22 +118,6 @@ typedef PipeCfg<2, 2, 2, 4, 3, 2, true> Pipe128x256;  // 4 waves, wave tile 64 x
 typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256;  // 8 waves, wave tile 64 x 128
 typedef PipeCfg<4, 2, 2, 3, 2, 2> Pipe256x192;  // narrow tiles of the mixed-width launch
 typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
-
-constexpr int kMaxDevices = 64;
-
-int device_cu_count(int* dev_out) {
-  static std::atomic<int> cached[kMaxDevices];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return -1;
-  *dev_out = dev;
-  if (dev < 0 || dev >= kMaxDevices) return 256;
-  int cus = cached[dev].load(std::memory_order_relaxed);
-  if (cus == 0) {
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-    cached[dev].store(cus, std::memory_order_relaxed);
-  }
-  return cus;
-}
 
 // Raise a kernel's dynamic LDS limit once per (kernel, device).
 template <class Kernel>
@@ -231,7 +234,6 @@ hipError_t launch_skinny(int mf, int nfs, int waves, int unroll, const Args& arg
   }
 }
 
-inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Makespan (in units of one 256 x 256 tile) of `ta` tiles of cost 1 followed by `tb` tiles of cost `cb`, handed
 // out in order, each to the worker that becomes free first.
@@ -406,7 +408,6 @@ struct Problem {
   hipStream_t stream;
 };
 
-bool misaligned(const void* ptr, size_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) != 0; }
 
 int run(const Problem& pr) {
   g_err[0] = '\0';

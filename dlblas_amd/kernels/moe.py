@@ -1,0 +1,47 @@
+"""MoE kernels of the FP8 expert MLP that sit next to the grouped GEMMs.
+
+``silu_and_mul_masked_post_quant_fwd`` is a drop-in for the reference function of the same name
+(dlblas/kernels/moe.py:264-319; kernel :204-261): same positional signature, same assertions, results written into
+the caller's ``output`` / ``output_scale``.  It runs between the two masked grouped GEMMs
+(dlblas/layers/moe/ep_moe.py:245-251).  Only quant_group_size 128 and float8_e4m3fn outputs are implemented.
+"""
+import torch
+
+from .. import _lib
+
+
+@torch.library.custom_op('dlblas::silu_and_mul_masked_post_quant', mutates_args=('output', 'output_scale'), device_types='cuda')
+def _masked_op(input: torch.Tensor, output: torch.Tensor, output_scale: torch.Tensor, masked_m: torch.Tensor) -> None:
+    G, M_max, two_n = input.shape
+    _lib.silu_mul_quant_masked(input, output, output_scale, masked_m, G, M_max, two_n // 2, output_scale.stride())
+
+
+def silu_and_mul_masked_post_quant_fwd(
+    input: torch.Tensor,
+    output: torch.Tensor,
+    output_scale: torch.Tensor,
+    quant_group_size: int,
+    masked_m: torch.Tensor,
+):
+    """input [E, M_max, 2N] (bf16 / fp16 / fp32) -> output [E, M_max, N] fp8 and output_scale [E, M_max, N / 128] fp32
+    for the first masked_m[e] tokens of every expert; other rows of both outputs keep their content."""
+    assert input.is_contiguous()
+    assert output.is_contiguous()
+    assert len(input.shape) == 3
+    assert input.shape[0] == masked_m.shape[0]
+    assert input.shape[-1] % 2 == 0
+    size_n = input.shape[-1] // 2
+    assert size_n % quant_group_size == 0
+    if quant_group_size != 128:
+        raise NotImplementedError(f'only quant_group_size 128 is implemented, got {quant_group_size}')
+    if output.dtype != torch.float8_e4m3fn:
+        raise NotImplementedError(f'only float8_e4m3fn output is implemented, got {output.dtype}')
+    if input.dtype not in _lib.IN_CODES:
+        raise TypeError(f'input must be bfloat16, float16 or float32, got {input.dtype}')
+    if tuple(output.shape) != (input.shape[0], input.shape[1], size_n):
+        raise ValueError(f'output shape {tuple(output.shape)} does not match input {tuple(input.shape)}')
+    if tuple(output_scale.shape) != (input.shape[0], input.shape[1], size_n // 128) or output_scale.dtype != torch.float32:
+        raise ValueError('output_scale must be float32 [E, M_max, N / 128]')
+    if masked_m.dtype != torch.int32:
+        masked_m = masked_m.to(torch.int32)
+    _masked_op(input, output, output_scale, masked_m.contiguous())

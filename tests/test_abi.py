@@ -1,4 +1,4 @@
-"""The C ABI library loads on a machine without a GPU and exports exactly what include/dlblas_fp8_gemm.h declares.
+"""The C ABI library loads on a machine without a GPU and exports exactly what the headers under include/ declare.
 No compute entry point is called with real work here."""
 import ctypes
 import os
@@ -12,8 +12,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, 'include', 'dlblas_fp8_gemm.h')
 
 
+HEADERS = [HEADER, os.path.join(ROOT, 'include', 'dlblas_fp8_moe.h')]
+
+
 def _declared_functions():
-    text = open(HEADER).read()
+    text = ''.join(open(h).read() for h in HEADERS)
     text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
     return sorted(set(re.findall(r'\b(dlb_[a-z0-9_]+)\s*\(', text)))
 

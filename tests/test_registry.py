@@ -167,7 +167,7 @@ def test_compat_aliases():
     import sys
 
     from dlblas_amd import compat
-    saved = {k: sys.modules.get(k) for k in list(compat._ALIASES) + ['deep_gemm']}
+    saved = {k: sys.modules.get(k) for k in list(compat._ALIASES) + ['deep_gemm', 'dlblas.layers', 'dlblas.layers.moe', 'dlblas.layers.moe.kernels']}
     try:
         compat.install()
         from dlblas.kernels.fp8_gemm import fp8_gemm
@@ -178,6 +178,11 @@ def test_compat_aliases():
                      'm_grouped_gemm_fp8_fp8_bf16_nt_contiguous', 'm_grouped_gemm_fp8_fp8_bf16_nt_masked'):
             assert hasattr(deep_gemm, name)
         assert deep_gemm.ceil_div(5, 4) == 2
+        from dlblas.kernels.moe import silu_and_mul_masked_post_quant_fwd
+        from dlblas.layers.moe.kernels.activation import silu_and_mul
+        from dlblas_amd.kernels import activation as act_mod, moe as moe_mod
+        assert silu_and_mul is act_mod.silu_and_mul
+        assert silu_and_mul_masked_post_quant_fwd is moe_mod.silu_and_mul_masked_post_quant_fwd
     finally:
         for k, v in saved.items():
             if v is None:
