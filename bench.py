@@ -311,6 +311,45 @@ def activation_workloads(dev):
     return rows
 
 
+def permutation_workloads(dev):
+    """ep_scatter / ep_gather at the expert-contiguous shape: 8192 tokens x top-8 over 256 experts of which 32 are
+    local (about one local slot per token), hidden 7168.  bytes = rows read + rows written (+ scales, tables)."""
+    import torch
+
+    from dlblas_amd import _lib
+    lib = _lib.load()
+    T, H, E, topk = 8192, 7168, 32, 8
+    gd = torch.Generator(device=dev).manual_seed(20)
+    x = torch.randint(0, 127, (T, H), device=dev, generator=gd, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    xs = torch.rand(T, H // 128, device=dev, generator=gd)
+    ids = torch.randint(0, 256, (T, topk), device=dev, generator=gd)
+    ids[ids >= E] = -1
+    wts = torch.rand(T, topk, device=dev, generator=gd)
+    routed = torch.bincount(ids[ids >= 0], minlength=E)
+    counts = ((routed + 127) // 128 * 128).to(torch.int32)
+    rows, n_routed = int(counts.sum()), int(routed.sum())
+    out = torch.empty(rows, H, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    out_s = torch.empty(rows, H // 128, device=dev)
+    m_indices = torch.empty(rows, dtype=torch.int32, device=dev)
+    out_idx = torch.empty_like(ids)
+    start = torch.empty(E, dtype=torch.int32, device=dev)
+    sargs = _lib.ep_scatter_args(x, xs, ids, counts, start, out, out_s, m_indices, out_idx)
+    _lib.check(lib.dlb_ep_scatter(*sargs))
+    ms = time_call(lambda: lib.dlb_ep_scatter(*sargs), 50, 5)
+    nbytes = (T + n_routed) * (H + 4 * (H // 128)) + 2 * 8 * T * topk + 4 * rows
+    res = [{'workload': f'ep_scatter_T{T}_top{topk}_E{E}_H{H}', 'routed_rows': n_routed, 'us_per_launch': ms * 1e3,
+            'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes}]
+    down = torch.randn(rows, H, device=dev, generator=gd).to(torch.bfloat16)
+    gout = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    gargs = _lib.ep_gather_args(down, ids, wts, out_idx, gout)
+    _lib.check(lib.dlb_ep_gather(*gargs))
+    ms = time_call(lambda: lib.dlb_ep_gather(*gargs), 50, 5)
+    nbytes = 2 * H * (n_routed + T) + (8 + 4 + 8) * T * topk
+    res.append({'workload': f'ep_gather_T{T}_top{topk}_H{H}_bf16', 'routed_rows': n_routed, 'us_per_launch': ms * 1e3,
+                'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes})
+    return res
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 --pmc runs kept under profiles/ (None when
     no counter run for this workload has been recorded)."""
@@ -399,6 +438,7 @@ def main():
         others += grouped_workloads(dev)
         others.append(quantiser_workload(dev))
         others += activation_workloads(dev)
+        others += permutation_workloads(dev)
         result['other_workloads'] = others
 
     if args.copy_calibration:

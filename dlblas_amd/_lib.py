@@ -39,6 +39,15 @@ SYMBOLS = {
     'dlb_silu_mul': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp] + [_c_i64] * 4 + [_c_vp]),
     'dlb_silu_mul_quant': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
     'dlb_silu_mul_quant_masked': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp, _c_vp] + [_c_i64] * 6 + [_c_vp]),
+    'dlb_ep_scatter_workspace_bytes': (_c_sz, [_c_i64, _c_i64, _c_i64]),
+    'dlb_ep_scatter':
+    (ctypes.c_int, [_c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_vp, _c_vp, ctypes.c_int, _c_vp,
+                    _c_i64, _c_vp, _c_i64, _c_i64, _c_vp, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
+                    _c_i64, _c_vp, _c_sz, _c_vp]),
+    'dlb_ep_gather':
+    (ctypes.c_int, [_c_vp, ctypes.c_int, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp, ctypes.c_int,
+                    _c_i64, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+    'dlb_scale_relayout': (ctypes.c_int, [_c_vp, _c_vp] + [_c_i64] * 5 + [_c_vp]),
 }
 
 _lock = threading.Lock()
@@ -228,3 +237,57 @@ def silu_mul_quant_masked(x, q, s, masked_m, G, M_max, N, s_strides):
     with torch.cuda.device(x.device):
         check(lib.dlb_silu_mul_quant_masked(_ptr(x), IN_CODES[x.dtype], _ptr(q), _ptr(s), _ptr(masked_m), G, M_max, N,
                                             s_strides[0], s_strides[1], s_strides[2], _stream(x)))
+
+
+IDX_CODES = {torch.int32: 0, torch.int64: 1}
+
+
+def _idx_code(t: torch.Tensor) -> int:
+    try:
+        return IDX_CODES[t.dtype]
+    except KeyError:
+        raise TypeError(f'index tensors must be int32 or int64, got {t.dtype}') from None
+
+
+def ep_scatter_args(recv_x, recv_x_scale, recv_topk, counts, expert_start_loc, out, out_scale, m_indices, output_index):
+    """Marshalled argument tuple of dlb_ep_scatter on the current stream (kept by callers that launch repeatedly)."""
+    lib = load()
+    _require_gpu(recv_x, recv_x_scale, recv_topk, counts, expert_start_loc, out, out_scale, m_indices, output_index)
+    T, H = recv_x.shape
+    topk = recv_topk.shape[1]
+    E = counts.shape[0]
+    stream, ws = _stream_and_ws(recv_x)
+    need = lib.dlb_ep_scatter_workspace_bytes(T, topk, E)
+    if need > ws.numel():
+        raise ValueError(f'ep_scatter needs {need} bytes of workspace, the per-stream buffer holds {ws.numel()}')
+    return (_ptr(recv_x), recv_x.stride(0), _ptr(recv_x_scale), recv_x_scale.stride(0), recv_x_scale.stride(1), _ptr(recv_topk),
+            _idx_code(recv_topk), recv_topk.stride(0), recv_topk.stride(1), _ptr(counts), _ptr(expert_start_loc),
+            _idx_code(expert_start_loc), _ptr(out), out.stride(0), _ptr(out_scale), out_scale.stride(0), out_scale.stride(1),
+            _ptr(m_indices), m_indices.numel(), _ptr(output_index), _idx_code(output_index), output_index.stride(0),
+            output_index.stride(1), T, H, topk, E, _ptr(ws), ws.numel(), ctypes.c_void_p(stream))
+
+
+def ep_scatter(recv_x, recv_x_scale, recv_topk, counts, expert_start_loc, out, out_scale, m_indices, output_index):
+    with torch.cuda.device(recv_x.device):
+        check(load().dlb_ep_scatter(*ep_scatter_args(recv_x, recv_x_scale, recv_topk, counts, expert_start_loc, out, out_scale,
+                                                     m_indices, output_index)))
+
+
+def ep_gather_args(inp, topk_ids, topk_weight, index, out):
+    _require_gpu(inp, topk_ids, topk_weight, index, out)
+    T, H = out.shape
+    return (_ptr(inp), IN_CODES[inp.dtype], inp.stride(0), _ptr(topk_ids), _idx_code(topk_ids), topk_ids.stride(0),
+            topk_ids.stride(1), _ptr(topk_weight), topk_weight.stride(0), topk_weight.stride(1), _ptr(index), _idx_code(index),
+            index.stride(0), index.stride(1), _ptr(out), IN_CODES[out.dtype], out.stride(0), T, H, topk_ids.shape[1], _stream(inp))
+
+
+def ep_gather(inp, topk_ids, topk_weight, index, out):
+    with torch.cuda.device(inp.device):
+        check(load().dlb_ep_gather(*ep_gather_args(inp, topk_ids, topk_weight, index, out)))
+
+
+def scale_relayout(src, dst, rows, kblocks, rows_pad):
+    lib = load()
+    _require_gpu(src, dst)
+    with torch.cuda.device(src.device):
+        check(lib.dlb_scale_relayout(_ptr(src), _ptr(dst), rows, kblocks, rows_pad, src.stride(0), src.stride(1), _stream(src)))

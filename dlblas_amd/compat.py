@@ -15,6 +15,8 @@ _ALIASES = {
     'dlblas.kernels.fp8_gemm': 'dlblas_amd.kernels.fp8_gemm',
     'dlblas.kernels.fp8': 'dlblas_amd.kernels.fp8',
     'dlblas.kernels.moe': 'dlblas_amd.kernels.moe',
+    'dlblas.kernels.fused_moe_v3': 'dlblas_amd.kernels.fused_moe_v3',
+    'dlblas.kernels.quant_dequant': 'dlblas_amd.kernels.quant_dequant',
     'dlblas.layers.moe.kernels.activation': 'dlblas_amd.kernels.activation',
     'dlblas.utils': 'dlblas_amd.utils',
     'dlblas.utils.logger': 'dlblas_amd.utils.logger',

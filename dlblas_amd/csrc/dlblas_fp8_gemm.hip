@@ -1,6 +1,7 @@
 // C ABI of the gfx950 FP8 block-scaled GEMM library: argument validation, kernel selection, launches.
 // The declarations and the contract of every entry point are in include/dlblas_fp8_gemm.h.
 #include "../../include/dlblas_fp8_gemm.h"
+#include "../../include/dlblas_fp8_moe.h"
 
 #include <atomic>
 #include <functional>
@@ -688,6 +689,27 @@ int dlb_fp8_gemm_tune(int knob, int value) {
 const char* dlb_fp8_gemm_variant_name(int variant) {
   if (variant < 0 || variant >= dlb::kVarCount) return nullptr;
   return dlb::kVariantNames[variant];
+}
+
+// declared in include/dlblas_fp8_moe.h; lives here next to the kernel it shares with the GEMM's own pre-pass
+int dlb_scale_relayout(const float* src, float* dst, int64_t rows, int64_t kblocks, int64_t rows_pad,
+                       int64_t src_stride_m, int64_t src_stride_k, void* stream) {
+  using namespace dlb;
+  clear_error();
+  if (rows < 0 || kblocks < 0 || rows_pad < rows)
+    return fail(DLB_ERR_BAD_SHAPE, "bad dimensions (rows=%lld kblocks=%lld rows_pad=%lld)", (long long)rows, (long long)kblocks,
+                (long long)rows_pad);
+  if (rows_pad == 0 || kblocks == 0) return DLB_OK;
+  if (!dst || (rows > 0 && !src)) return fail(DLB_ERR_NULL_POINTER, "src or dst is NULL");
+  if (rows_pad >= (1ll << 31) || kblocks >= (1ll << 31) || ceil_div(kblocks, 32) > 65535)
+    return fail(DLB_ERR_BAD_SHAPE, "dimensions beyond the supported range");
+  const dim3 grid(static_cast<unsigned>(ceil_div(rows_pad, 32)), static_cast<unsigned>(ceil_div(kblocks, 32)), 1);
+  hipLaunchKernelGGL(fp8_scale_transpose_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), src, dst,
+                     static_cast<int>(rows), static_cast<int>(kblocks), static_cast<int>(rows_pad), static_cast<int64_t>(0),
+                     src_stride_m, src_stride_k);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "scale_relayout launch failed: %s", hipGetErrorString(e));
+  return DLB_OK;
 }
 
 }  // extern "C"

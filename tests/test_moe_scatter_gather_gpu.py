@@ -1,0 +1,233 @@
+"""GPU parity of ep_scatter / ep_gather / tma_align_input_scale / fused_moe_v3 (Python entry points -> C ABI) against
+oracle/moe_scatter_gather.py.  Index and byte work is compared bit for bit; the gather's fp32 FMA chain is compared
+with the oracle's (fp64-evaluated) chain: equal after the cast except where the fp32 sum sits on a rounding boundary."""
+import pytest
+import torch
+
+import helpers
+from oracle import fp8_block_gemm as orc
+from oracle import moe_activation as act
+from oracle import moe_scatter_gather as sg
+from test_oracle_moe_scatter_gather import reference_test_routing, scatter_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module')
+def dev():
+    from dlblas_amd import _lib
+    _lib.load()
+    return torch.device('cuda:0')
+
+
+def _scatter_both(dev, c, start_dtype=torch.int64, fill=0x33, strided_topk=False):
+    from dlblas_amd.kernels.fused_moe_v3 import ep_scatter
+    rows, H = c['all_tokens'], c['x'].shape[1]
+
+    def fresh(device):
+        out = torch.full((rows, H), fill, dtype=torch.uint8, device=device).view(torch.float8_e4m3fn)
+        out_s = torch.full((rows, H // 128), -5.0, device=device)
+        m_indices = torch.full((rows, ), -9, dtype=torch.int32, device=device)
+        out_idx = torch.full_like(c['ids'], -1).to(device)
+        start = torch.full((c['E'], ), -1, dtype=start_dtype, device=device)
+        return out, out_s, m_indices, out_idx, start
+
+    ref = fresh('cpu')
+    sg.ep_scatter_ref(c['x'], c['xs'], c['ids'], c['counts'], ref[4], ref[0], ref[1], ref[2], ref[3])
+    got = fresh(dev)
+    ids = c['ids'].to(dev)
+    if strided_topk:
+        wide = torch.full((ids.shape[0], ids.shape[1] * 2), -1, dtype=ids.dtype, device=dev)
+        wide[:, ::2] = ids
+        ids = wide[:, ::2]
+    ep_scatter(c['x'].to(dev), c['xs'].to(dev), ids, c['counts'].to(dev), got[4], got[0], got[1], got[2], got[3])
+    torch.cuda.synchronize()
+    return ref, got
+
+
+def _assert_scatter_equal(ref, got):
+    assert torch.equal(got[0].cpu().view(torch.uint8), ref[0].view(torch.uint8)), 'output_tensor'
+    assert torch.equal(got[1].cpu(), ref[1]), 'output_tensor_scale'
+    assert torch.equal(got[2].cpu(), ref[2]), 'm_indices'
+    assert torch.equal(got[3].cpu(), ref[3]), 'output_index'
+    assert torch.equal(got[4].cpu(), ref[4]), 'expert_start_loc'
+
+
+def test_scatter_reference_test_construction(dev):
+    """tests/kernels/test_scatter_gather.py:10-76: 7 tokens, hidden 4096, 32 experts of which 6-8 hold 128 rows each,
+    int32 ids, int64 expert_start_loc."""
+    for seed in range(3):
+        print(f'case scatter reference construction seed={seed}', flush=True)
+        c = scatter_case(seed)
+        ref, got = _scatter_both(dev, c)
+        _assert_scatter_equal(ref, got)
+        # the reference test's own assertions
+        m_ref = torch.repeat_interleave(torch.arange(32, dtype=torch.int32), c['counts'].long())
+        assert torch.equal(got[2].cpu(), m_ref)
+        idx = got[3].cpu()
+        for i in range(7):
+            for j in range(8):
+                if c['ids'][i, j] >= 0:
+                    assert torch.equal(got[0][int(idx[i, j])].cpu().view(torch.uint8), c['x'][i].view(torch.uint8))
+                    assert torch.equal(got[1][int(idx[i, j])].cpu(), c['xs'][i])
+
+
+@pytest.mark.parametrize('index_dtype,start_dtype,strided', [(torch.int64, torch.int32, False), (torch.int32, torch.int64, True)])
+@pytest.mark.parametrize('T,H,E,topk', [(1, 128, 1, 1), (300, 1024, 8, 8), (1000, 7168, 32, 8), (257, 256, 40, 3), (50, 512, 300, 64)])
+def test_scatter_matches_oracle(dev, T, H, E, topk, index_dtype, start_dtype, strided):
+    print(f'case scatter T={T} H={H} E={E} topk={topk} {index_dtype} {start_dtype} strided={strided}', flush=True)
+    g = helpers.gen(T + H + E)
+    ids = torch.randint(-1, E, (T, topk), generator=g).to(index_dtype)       # -1 = no expert
+    ids[torch.rand(T, topk, generator=g) < 0.2] = -1
+    if E > 2:
+        ids[0, 0] = E + 5                                                       # beyond the table: skipped
+    routed = torch.bincount(ids[(ids >= 0) & (ids < E)].long(), minlength=E)
+    counts = ((routed + 127) // 128 * 128).to(torch.int32)
+    c = dict(x=torch.randn(T, H, generator=g).to(torch.float8_e4m3fn), xs=torch.randn(T, H // 128, generator=g), ids=ids,
+             counts=counts, all_tokens=int(counts.sum()), E=E)
+    ref, got = _scatter_both(dev, c, start_dtype=start_dtype, strided_topk=strided)
+    _assert_scatter_equal(ref, got)
+
+
+def test_scatter_full_size_properties(dev):
+    """8192 tokens x top-8 over 32 experts, hidden 7168 (the expert-contiguous workload): properties that need no
+    CPU pass over the data - every routed slot finds its row, rows are a bijection, m_indices is sorted."""
+    from dlblas_amd.kernels.fused_moe_v3 import ep_scatter
+    print('case scatter full size', flush=True)
+    T, H, E, topk = 8192, 7168, 32, 8
+    gd = torch.Generator(device=dev).manual_seed(20)
+    x = torch.randint(0, 256, (T, H), device=dev, generator=gd, dtype=torch.uint8)
+    x[x == 0x7f] = 0
+    x[x == 0xff] = 0
+    xs = torch.rand(T, H // 128, device=dev, generator=gd)
+    ids = torch.randint(0, 256, (T, topk), device=dev, generator=gd)  # 256 global experts, 32 of them local
+    ids[ids >= E] = -1
+    routed = torch.bincount(ids[ids >= 0], minlength=E)
+    counts = ((routed + 127) // 128 * 128).to(torch.int32)
+    rows = int(counts.sum())
+    out = torch.zeros(rows, H, dtype=torch.uint8, device=dev)
+    out_s = torch.full((rows, H // 128), -1.0, device=dev)
+    m_indices = torch.empty(rows, dtype=torch.int32, device=dev)
+    out_idx = torch.full_like(ids, -1)
+    start = torch.empty(E, dtype=torch.int32, device=dev)
+    ep_scatter(x.view(torch.float8_e4m3fn), xs, ids, counts, start, out.view(torch.float8_e4m3fn), out_s, m_indices, out_idx)
+    torch.cuda.synchronize()
+    valid = ids >= 0
+    dst = out_idx[valid]
+    assert dst.numel() == int(routed.sum()) and torch.unique(dst).numel() == dst.numel()
+    tok = torch.arange(T, device=dev).unsqueeze(1).expand(T, topk)[valid]
+    assert torch.equal(out[dst], x[tok]) and torch.equal(out_s[dst], xs[tok])
+    assert torch.equal(m_indices[dst].long(), ids[valid])
+    assert torch.equal(m_indices, torch.repeat_interleave(torch.arange(E, device=dev, dtype=torch.int32), counts.long()))
+    excl = torch.cumsum(counts.long(), 0) - counts.long()
+    assert torch.equal(start.long(), excl + routed)
+    assert (out_idx[~valid] == -1).all()
+    # token-major order inside an expert
+    for e in (0, 17, 31):
+        d = out_idx[ids == e]
+        assert torch.equal(d, torch.arange(int(excl[e]), int(excl[e]) + d.numel(), device=dev))
+
+
+@pytest.mark.parametrize('in_dtype,out_dtype', [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32),
+                                                (torch.float16, torch.bfloat16)])
+@pytest.mark.parametrize('T,H,topk,rows', [(7, 4096, 8, 384), (1, 8, 1, 4), (333, 7168, 8, 2000), (40, 1024, 64, 77)])
+def test_gather_matches_oracle(dev, T, H, topk, rows, in_dtype, out_dtype):
+    from dlblas_amd.kernels.fused_moe_v3 import ep_gather
+    print(f'case gather T={T} H={H} topk={topk} {in_dtype}->{out_dtype}', flush=True)
+    g = helpers.gen(T * 7 + H)
+    ids = torch.randint(-1, 5, (T, topk), generator=g, dtype=torch.int32)
+    if T > 2:
+        ids[1] = -1                                             # a token without any expert: zeros
+    w = torch.rand(T, topk, generator=g)
+    index = torch.randint(0, rows, (T, topk), generator=g, dtype=torch.int32)
+    inp = torch.randn(rows, H, generator=g).to(in_dtype)
+    ref = torch.full((T, H), 3.0, dtype=out_dtype)
+    sg.ep_gather_ref(inp, ids, w, index, ref)
+    out = torch.full((T, H), 3.0, dtype=out_dtype, device=dev)
+    ep_gather(inp.to(dev), ids.to(dev), w.to(dev), index.to(dev), out)
+    torch.cuda.synchronize()
+    o, r = out.cpu().float(), ref.float()
+    ulp = {torch.bfloat16: 2**-7, torch.float16: 2**-10, torch.float32: 2**-22}[out_dtype]
+    assert ((o - r).abs() <= r.abs() * ulp + 1e-30).all()
+    assert int((o != r).sum()) <= max(3, 1e-4 * o.numel())
+    if T > 2:
+        assert (out[1] == 0).all()
+
+
+def test_gather_reference_test_construction(dev):
+    """tests/kernels/test_scatter_gather.py:79-107 (int32 ids, weights k / 10, all-zero input) plus the same tables
+    on a random input."""
+    from dlblas_amd.kernels.fused_moe_v3 import ep_gather
+    print('case gather reference construction', flush=True)
+    ids, w = reference_test_routing(3)
+    index = torch.zeros_like(ids)
+    zero_in = torch.zeros(384, 4096, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(7, 4096, dtype=torch.bfloat16, device=dev)
+    ep_gather(zero_in, ids.to(dev), w.to(dev), index.to(dev), out)
+    torch.cuda.synchronize()
+    assert torch.allclose(out.cpu(), torch.zeros(7, 4096, dtype=torch.bfloat16), atol=1e-2, rtol=0)
+
+
+def test_tma_align_input_scale(dev):
+    from dlblas_amd.kernels.quant_dequant import get_tma_aligned_size, tma_align_input_scale
+    print('case scale relayout', flush=True)
+    g = helpers.gen(2)
+    for m, k in ((1, 1), (7, 56), (130, 16), (9728, 56), (33, 70)):
+        s = torch.randn(m, k, generator=g)
+        out = tma_align_input_scale(s.to(dev))
+        torch.cuda.synchronize()
+        ref = sg.tma_align_input_scale_ref(s)
+        assert tuple(out.shape) == (m, k) and out.stride() == ref.stride() == (1, get_tma_aligned_size(m, 4))
+        assert torch.equal(out.cpu(), ref)
+    # a column-major input view is accepted as well
+    s = torch.randn(16, 40, generator=g).t()
+    assert torch.equal(tma_align_input_scale(s.to(dev)).cpu(), s)
+
+
+def test_fused_moe_v3_end_to_end(dev):
+    """scatter -> GEMM -> silu*up + quant -> GEMM -> gather against the same chain of oracles.  The device's GEMM
+    differs from the oracle's within the GEMM tolerance, which the quantiser between the GEMMs can turn into a
+    different fp8 code here and there; the bar is the reference's similarity metric plus a bound on the largest
+    deviation relative to the output's rms."""
+    from dlblas_amd.kernels.fused_moe_v3 import fused_moe_v3
+    print('case fused_moe_v3', flush=True)
+    T, K, N, E, topk = 96, 512, 1024, 4, 2  # N = gate + up
+    g = helpers.gen(77)
+    x = torch.randn(T, K, generator=g).to(torch.bfloat16)
+    x_q, x_s = orc.quant_act_1x128(x)
+    w13, w13_s, w2, w2_s = [], [], [], []
+    for _ in range(E):
+        q, s = orc.quant_weight_128x128((torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16))
+        w13.append(q), w13_s.append(s)
+        q, s = orc.quant_weight_128x128((torch.randn(K, N // 2, generator=g) * 0.05).to(torch.bfloat16))
+        w2.append(q), w2_s.append(s)
+    w13, w13_s, w2, w2_s = torch.stack(w13), torch.stack(w13_s), torch.stack(w2), torch.stack(w2_s)
+    ids = torch.stack([torch.randperm(E + 2, generator=g)[:topk] - 2 for _ in range(T)]).long()  # -2, -1: elsewhere
+    wts = torch.rand(T, topk, generator=g)
+    routed = torch.bincount(ids[ids >= 0], minlength=E)
+    counts = [int(v) for v in (routed + 127) // 128 * 128]
+    out = fused_moe_v3((x_q.to(dev), x_s.to(dev)), ids.to(dev), wts.to(dev), (w13.to(dev), w13_s.to(dev)),
+                       (w2.to(dev), w2_s.to(dev)), counts)
+    torch.cuda.synchronize()
+    # oracle chain
+    rows = sum(counts)
+    inp = torch.zeros(rows, K, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    inp_s = torch.zeros(rows, K // 128)
+    m_indices = torch.empty(rows, dtype=torch.int32)
+    out_idx = torch.full_like(ids, -1)
+    start = torch.zeros(E, dtype=torch.int32)
+    sg.ep_scatter_ref(x_q, x_s, ids, torch.tensor(counts, dtype=torch.int32), start, inp, inp_s, m_indices, out_idx)
+    gateup = torch.zeros(rows, N, dtype=torch.bfloat16)
+    orc.grouped_contiguous_ref(inp, inp_s, w13, w13_s, gateup, m_indices)
+    d_q, d_s = act.silu_and_mul_post_quant_ref(gateup)
+    down = torch.zeros(rows, K, dtype=torch.bfloat16)
+    orc.grouped_contiguous_ref(d_q, d_s, w2, w2_s, down, m_indices)
+    ref = torch.zeros(T, K, dtype=torch.bfloat16)
+    sg.ep_gather_ref(down, ids, wts, out_idx, ref)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (T, K)
+    o, r = out.cpu().float(), ref.float()
+    assert orc.similarity_gap(o, r) <= 1e-4
+    assert (o - r).abs().max() <= 0.05 * r.pow(2).mean().sqrt()
+    # the two early exits of the reference driver (fused_moe_v3.py:255-259)
+    assert torch.equal(fused_moe_v3((x_q.to(dev), x_s.to(dev)), ids.to(dev), wts.to(dev), None, None, None).cpu(),
+                       x_q.to(torch.bfloat16))
