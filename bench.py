@@ -266,8 +266,19 @@ def quantiser_workload(dev):
             vp(torch.cuda.current_stream().cuda_stream))
     ms = time_call(lambda: lib.dlb_fp8_quant_1x128(*args), 100, 10)
     nbytes = 2 * M * K + M * K + 4 * M * (K // 128)
-    return {'workload': f'quant_1x128_bf16_{M}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
-            'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes}
+    row = {'workload': f'quant_1x128_bf16_{M}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
+           'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes}
+    # the producer of (b, b_s): 128 x 128 block quantisation of a bf16 [7168, 18432] weight
+    from dlblas_amd.kernels.fp8 import per_block_quant_fp8
+    N = 7168
+    w = (torch.randn(N, K, device=dev, generator=torch.Generator(device=dev).manual_seed(21)) * 0.02).to(torch.bfloat16)
+    w_q, w_s = per_block_quant_fp8(w)
+    wargs = (vp(w.data_ptr()), _lib.IN_CODES[w.dtype], vp(w_q.data_ptr()), vp(w_s.data_ptr()), 1, N, K, K, 1e-10,
+             vp(torch.cuda.current_stream().cuda_stream))
+    ms = time_call(lambda: lib.dlb_fp8_quant_128x128(*wargs), 50, 5)
+    nbytes = 2 * N * K + N * K + 4 * (N // 128) * (K // 128)
+    return [row, {'workload': f'quant_128x128_bf16_{N}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
+                  'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes}]
 
 
 def activation_workloads(dev):
@@ -436,7 +447,7 @@ def main():
                             'note': '24 distinct weight copies in rotation (353 MB) so reads miss the 256 MB cache'}
         log('grouped workloads')
         others += grouped_workloads(dev)
-        others.append(quantiser_workload(dev))
+        others += quantiser_workload(dev)
         others += activation_workloads(dev)
         others += permutation_workloads(dev)
         result['other_workloads'] = others

@@ -33,6 +33,7 @@ SYMBOLS = {
     'dlb_fp8_gemm_grouped_masked':
     (ctypes.c_int, [_c_vp] * 6 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 3 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_quant_1x128': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
+    'dlb_fp8_quant_128x128': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 4 + [ctypes.c_float, _c_vp]),
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
     'dlb_fp8_gemm_tune': (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
@@ -291,3 +292,11 @@ def scale_relayout(src, dst, rows, kblocks, rows_pad):
     _require_gpu(src, dst)
     with torch.cuda.device(src.device):
         check(lib.dlb_scale_relayout(_ptr(src), _ptr(dst), rows, kblocks, rows_pad, src.stride(0), src.stride(1), _stream(src)))
+
+
+def quant_128x128(w3d, q, s, G, N, K, eps):
+    lib = load()
+    _require_gpu(w3d, q, s)
+    with torch.cuda.device(w3d.device):
+        check(lib.dlb_fp8_quant_128x128(_ptr(w3d), IN_CODES[w3d.dtype], _ptr(q), _ptr(s), G, N, K, w3d.stride(-2), float(eps),
+                                        _stream(w3d)))

@@ -673,6 +673,37 @@ int dlb_fp8_quant_1x128(const void* x, int x_dtype, void* q, float* s, int64_t r
   return DLB_OK;
 }
 
+int dlb_fp8_quant_128x128(const void* w, int w_dtype, void* q, float* s, int64_t G, int64_t N, int64_t K,
+                          int64_t w_row_stride, float eps, void* stream) {
+  using namespace dlb;
+  g_err[0] = '\0';
+  if (w_dtype < kInBf16 || w_dtype > kInF32) return fail(DLB_ERR_BAD_DTYPE, "w_dtype %d is not DLB_IN_BF16 / F16 / F32", w_dtype);
+  if (G < 0 || N < 0 || K < 0)
+    return fail(DLB_ERR_BAD_SHAPE, "negative dimension (G=%lld N=%lld K=%lld)", (long long)G, (long long)N, (long long)K);
+  if (K % 8 != 0) return fail(DLB_ERR_BAD_SHAPE, "K=%lld is not a multiple of 8", (long long)K);
+  if (G == 0 || N == 0 || K == 0) return DLB_OK;
+  if (!w || !q || !s) return fail(DLB_ERR_NULL_POINTER, "w, q or s is NULL");
+  const int64_t esz = w_dtype == kInF32 ? 4 : 2;
+  if (w_row_stride < K) return fail(DLB_ERR_BAD_STRIDE, "w row stride %lld < K", (long long)w_row_stride);
+  if (misaligned(w, 16) || (w_row_stride * esz) % 16 != 0 || misaligned(q, 8) || misaligned(s, 4))
+    return fail(DLB_ERR_ALIGNMENT, "w rows must be 16-byte aligned, q 8-byte aligned");
+  const int64_t nbn = ceil_div(N, kScaleBlock), nbk = ceil_div(K, kScaleBlock);
+  const int64_t blocks = G * nbn * nbk;
+  if (blocks >= (1ll << 31) || nbn >= (1ll << 30) || nbk >= (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many blocks");
+  BlockQuantArgs a{w, static_cast<uint8_t*>(q), s, N, K, w_row_stride, static_cast<int>(nbn), static_cast<int>(nbk), eps};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+  if (w_dtype == kInBf16)
+    hipLaunchKernelGGL(fp8_quant_128x128_kernel<kInBf16>, grid, block, 0, st, a);
+  else if (w_dtype == kInF16)
+    hipLaunchKernelGGL(fp8_quant_128x128_kernel<kInF16>, grid, block, 0, st, a);
+  else
+    hipLaunchKernelGGL(fp8_quant_128x128_kernel<kInF32>, grid, block, 0, st, a);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return DLB_OK;
+}
+
 int dlb_fp8_gemm_force_variant(int variant) {
   if (variant >= dlb::kVarCount) return dlb::fail(DLB_ERR_BAD_SHAPE, "unknown kernel variant %d", variant);
   dlb::g_forced_variant = variant < 0 ? -1 : variant;

@@ -121,4 +121,75 @@ __global__ void __launch_bounds__(256) fp8_quant_1x128_kernel(const QuantArgs p)
   }
 }
 
+// 128 x 128 block quantiser for weights: one scale per block, s = max(amax, eps) / 448, same cast as above.  The
+// reference ships no such function; the scheme is that of its test data builder
+// (tests/kernels/test_fused_moe_v2.py:35-60) and of the b_s operand of fp8_gemm (dlblas/kernels/fp8_gemm.py:47).
+// One workgroup per block: 8 chunks of 8 elements per thread stay in registers between the amax reduction and the
+// cast, so every element is read once.  Blocks at the N and K edges are ragged; K % 8 == 0, rows 16-byte aligned.
+struct BlockQuantArgs {
+  const void* w;  // [G][N][K], row stride w_row_stride, group stride N * w_row_stride (elements)
+  uint8_t* q;     // [G][N][K] contiguous
+  float* s;       // [G][ceil(N/128)][ceil(K/128)] contiguous
+  int64_t N, K, w_row_stride;
+  int nblocks_n, nblocks_k;
+  float eps;
+};
+
+template <int IN>
+__global__ void __launch_bounds__(256) fp8_quant_128x128_kernel(const BlockQuantArgs p) {
+  __shared__ float wave_max[4];
+  const int tid = threadIdx.x;
+  const int64_t blk = blockIdx.x;
+  const int kb = static_cast<int>(blk % p.nblocks_k);
+  const int64_t rest = blk / p.nblocks_k;
+  const int nb = static_cast<int>(rest % p.nblocks_n);
+  const int64_t g = rest / p.nblocks_n;
+  const void* w_g = static_cast<const char*>(p.w) + g * p.N * p.w_row_stride * (IN == kInF32 ? 4 : 2);
+  uint8_t* q_g = p.q + g * p.N * p.K;
+  float v[8][8];
+  bool live[8];
+  float amax = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = tid + 256 * k;  // chunk of the block: row i / 16, columns 8 (i % 16) ..
+    const int64_t row = static_cast<int64_t>(nb) * 128 + (i >> 4);
+    const int64_t col = static_cast<int64_t>(kb) * 128 + (i & 15) * 8;
+    live[k] = row < p.N && col < p.K;
+    if (live[k]) {
+      quant_load8<IN>(w_g, row * p.w_row_stride + col, v[k]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[k][j] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[k][j]));
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+  if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+  const float scale = fmaxf(amax, p.eps) / 448.0f;
+  const float inv_scale = 1.0f / scale;
+  if (tid == 0) p.s[(g * p.nblocks_n + nb) * p.nblocks_k + kb] = scale;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    if (!live[k]) continue;
+    const int i = tid + 256 * k;
+    const int64_t row = static_cast<int64_t>(nb) * 128 + (i >> 4);
+    const int64_t col = static_cast<int64_t>(kb) * 128 + (i & 15) * 8;
+    int packed[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      float c[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) c[j] = fminf(fmaxf(div_by_scale(v[k][4 * h + j], scale, inv_scale), -448.0f), 448.0f);
+      int wd = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], 0, false);
+      wd = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], wd, true);
+      packed[h] = wd;
+    }
+    *reinterpret_cast<v2i*>(q_g + row * p.K + col) = v2i{packed[0], packed[1]};
+  }
+}
+
 }  // namespace dlb

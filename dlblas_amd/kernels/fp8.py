@@ -61,6 +61,39 @@ def per_token_group_quant_fp8(
     return x_q, x_s
 
 
+@torch.library.custom_op('dlblas::per_block_quant_fp8', mutates_args=('w_q', 'w_s'), device_types='cuda')
+def block_quant_op(w: torch.Tensor, w_q: torch.Tensor, w_s: torch.Tensor, eps: float) -> None:
+    G = w.shape[0] if w.dim() == 3 else 1
+    _lib.quant_128x128(w, w_q, w_s, G, w.shape[-2], w.shape[-1], eps)
+
+
+def per_block_quant_fp8(w: torch.Tensor, block_size: int = 128, eps: float = 1e-10,
+                        dtype: Optional[torch.dtype] = torch.float8_e4m3fn) -> Tuple[torch.Tensor, torch.Tensor]:
+    """128 x 128 block quantisation of a weight ``w`` [N, K] or [G, N, K] to float8_e4m3fn: the (b, b_s) operands of
+    fp8_gemm (dlblas/kernels/fp8_gemm.py:47,74-76) and of the grouped GEMMs.  The reference has no such function;
+    the scheme is that of its test data builder (tests/kernels/test_fused_moe_v2.py:35-60).
+
+    Returns ``(w_q, w_s)``: ``w_q`` like ``w`` in fp8, ``w_s`` fp32 ``[(G,) ceil(N/128), ceil(K/128)]``.
+    """
+    if block_size != 128:
+        raise NotImplementedError(f'only block_size 128 is implemented, got {block_size}')
+    if dtype != torch.float8_e4m3fn:
+        raise NotImplementedError(f'only float8_e4m3fn is implemented, got {dtype}')
+    if w.dtype not in _lib.IN_CODES:
+        raise TypeError(f'w must be bfloat16, float16 or float32, got {w.dtype}')
+    if w.dim() not in (2, 3):
+        raise ValueError('w must be [N, K] or [G, N, K]')
+    assert w.stride(-1) == 1, 'the last dimension of w must be contiguous'
+    if w.dim() == 3 and w.stride(0) != w.shape[1] * w.stride(1):
+        w = w.contiguous()
+    N, K = w.shape[-2], w.shape[-1]
+    assert K % 8 == 0, f'K {K} must be a multiple of 8'
+    w_q = torch.empty(w.shape, device=w.device, dtype=dtype)
+    w_s = torch.empty(w.shape[:-2] + (-(-N // 128), -(-K // 128)), device=w.device, dtype=torch.float32)
+    block_quant_op(w, w_q, w_s, float(eps))
+    return w_q, w_s
+
+
 def _bench(x, group_size, warmup: int = 3, rep: int = 10) -> float:
     for _ in range(warmup):
         per_token_group_quant_fp8(x, group_size)

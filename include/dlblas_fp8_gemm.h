@@ -164,6 +164,21 @@ int dlb_fp8_quant_1x128(const void* x, int x_dtype, void* q, float* s, int64_t r
                         int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream);
 
 /*
+ * 128 x 128 block quantiser, the producer of (b, b_s): one scale per block of the weight matrix, blocks at the N and
+ * K edges ragged.  The reference has no such function in the package; the scheme (block amax / 448) is that of its
+ * test data builder (tests/kernels/test_fused_moe_v2.py:35-60) and of the b_s operand of fp8_gemm
+ * (dlblas/kernels/fp8_gemm.py:47):
+ *     s[g, i, j] = max(max |w[g, 128 i .., 128 j ..]|, eps) / 448,   q = round_to_nearest_even_e4m3(clamp(w / s, -448, 448))
+ *
+ *   w  [G, N, K]                        bf16 / fp16 / fp32 (w_dtype), K contiguous, row stride w_row_stride elements,
+ *                                       experts N * w_row_stride apart, rows 16-byte aligned, K % 8 == 0
+ *   q  [G, N, K]                        e4m3fn, contiguous
+ *   s  [G, ceil(N/128), ceil(K/128)]    fp32, contiguous
+ */
+int dlb_fp8_quant_128x128(const void* w, int w_dtype, void* q, float* s, int64_t G, int64_t N, int64_t K,
+                          int64_t w_row_stride, float eps, void* stream);
+
+/*
  * Tuning / test hook: force the kernel variant the next calls FROM THIS THREAD use.
  * variant < 0 restores the built-in shape heuristic.  Returns DLB_ERR_BAD_SHAPE for an unknown id.
  * Variant ids are listed by dlb_fp8_gemm_variant_name().

@@ -100,3 +100,62 @@ def test_quant_feeds_the_gemm(dev):
         torch.set_default_dtype(prev)
     a_q_ref, a_s_ref = orc.quant_act_1x128(a)
     helpers.tolerance_check(out, orc.dequant_ref(a_q_ref, a_s_ref, b_q, b_s), 'quant + gemm')
+
+
+def _check_block(w_cpu, dev):
+    from dlblas_amd.kernels.fp8 import per_block_quant_fp8
+    if w_cpu.dim() == 2:
+        q_ref, s_ref = orc.quant_weight_128x128(w_cpu)
+    else:
+        qs = [orc.quant_weight_128x128(w_cpu[i]) for i in range(w_cpu.shape[0])]
+        q_ref, s_ref = torch.stack([q for q, _ in qs]), torch.stack([s for _, s in qs])
+    q, s = per_block_quant_fp8(w_cpu.to(dev))
+    torch.cuda.synchronize()
+    assert q.dtype == torch.float8_e4m3fn and q.shape == w_cpu.shape and tuple(s.shape) == tuple(s_ref.shape)
+    assert torch.equal(s.cpu(), s_ref), 'scales differ'
+    qb, rb = q.cpu().view(torch.uint8), q_ref.view(torch.uint8)
+    same = (qb == rb) | (((qb & 0x7F) == 0) & ((rb & 0x7F) == 0))
+    assert bool(same.all()), f'{int((~same).sum())} of {same.numel()} codes differ'
+    return q, s
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize('shape', [(128, 128), (2112, 7168), (300, 392), (1, 8), (3, 200, 264), (4, 512, 1024)])
+def test_block_quant_matches_oracle_bit_for_bit(dev, dtype, shape):
+    """128 x 128 weight blocks, ragged at the N and K edges, 2-d and per-expert 3-d."""
+    print(f'case block quant {dtype} {shape}', flush=True)
+    g = helpers.gen(41)
+    w = (torch.randn(*shape, generator=g) * 0.02).to(dtype)
+    _check_block(w, dev)
+
+
+def test_block_quant_edge_values_and_feeds_the_gemm(dev):
+    from dlblas_amd.kernels.fp8_gemm import fp8_gemm
+    print('case block quant edges', flush=True)
+    w = torch.zeros(256, 256, dtype=torch.bfloat16)
+    w[:128, :128] = 0                      # all-zero block: eps scale, zero codes
+    w[128:, :128] = 3.0                    # constant block: every code is 448
+    w[:128, 128:] = torch.linspace(-1, 1, 128 * 128).reshape(128, 128).to(torch.bfloat16)
+    w[128:, 128:] = 1e-30                  # far below eps
+    q, s = _check_block(w, dev)
+    assert s[0, 0] == torch.tensor(1e-10, dtype=torch.float32) / 448
+    assert (orc.decode_e4m3fn(q[128:, :128].cpu()) == 448).all()
+    # the quantised weight is a valid b / b_s operand
+    g = helpers.gen(43)
+    wb = (torch.randn(384, 1024, generator=g) * 0.02).to(torch.bfloat16)
+    a_q, a_s = orc.quant_act_1x128(torch.randn(64, 1024, generator=g).to(torch.bfloat16))
+    b_q, b_s = _check_block(wb, dev)
+    out = fp8_gemm(a_q.to(dev), b_q, a_s.to(dev), b_s)
+    torch.cuda.synchronize()
+    helpers.tolerance_check(out, orc.dequant_ref(a_q, a_s, b_q.cpu(), b_s.cpu()), 'gemm on device-quantised weights')
+
+
+def test_block_quant_asserts(dev):
+    from dlblas_amd.kernels.fp8 import per_block_quant_fp8
+    w = torch.zeros(128, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(NotImplementedError):
+        per_block_quant_fp8(w, 64)
+    with pytest.raises(AssertionError):
+        per_block_quant_fp8(torch.zeros(128, 132, dtype=torch.bfloat16, device=dev)[:, :4])
+    with pytest.raises(ValueError):
+        per_block_quant_fp8(torch.zeros(128, dtype=torch.bfloat16, device=dev))
