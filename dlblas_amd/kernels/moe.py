@@ -45,3 +45,39 @@ def silu_and_mul_masked_post_quant_fwd(
     if masked_m.dtype != torch.int32:
         masked_m = masked_m.to(torch.int32)
     _masked_op(input, output, output_scale, masked_m.contiguous())
+
+
+def low_latency_experts(
+    hidden_states_fp8,
+    gate_up_weight: torch.Tensor,
+    gate_up_scale: torch.Tensor,
+    gate_down_weight: torch.Tensor,
+    gate_down_scale: torch.Tensor,
+    masked_m: torch.Tensor,
+    expected_m: int,
+    out_dtype: torch.dtype = torch.bfloat16,
+    block_size: int = 128,
+):
+    """The per-GPU compute of the decode MoE layer, ``FusedMoELowLatency.experts`` of the reference
+    (dlblas/layers/moe/ep_moe.py:199-261) without its dispatch / combine: masked grouped GEMM (gate and up) ->
+    silu * up + 1 x 128 quantisation of the valid rows -> masked grouped GEMM (down).
+
+    hidden_states_fp8 = (a [G, M_max, K] fp8, a_s [G, M_max, K / 128] fp32); weights [G, N, K] / [G, K, N / 2] fp8 with
+    128 x 128 block scales; masked_m [G] int32.  Returns down_output [G, M_max, K] in out_dtype; rows at or beyond
+    masked_m[g] are not written (they hold whatever the allocation held, as in the reference).
+    """
+    from .fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
+    a, a_s = hidden_states_fp8
+    num_groups, m, k = a.shape
+    n = gate_up_weight.size(1)
+    expected_m = min(expected_m, m)
+    gateup_output = torch.empty((num_groups, m, n), device=a.device, dtype=out_dtype)
+    m_grouped_fp8_gemm_nt_masked((a, a_s), (gate_up_weight, gate_up_scale), gateup_output, masked_m, expected_m)
+    down_input = torch.empty((num_groups, m, n // 2), device=a.device, dtype=gate_down_weight.dtype)
+    down_input_scale = torch.empty((num_groups, m, n // 2 // block_size), device=a.device, dtype=torch.float32)
+    silu_and_mul_masked_post_quant_fwd(gateup_output, down_input, down_input_scale, block_size, masked_m)
+    del gateup_output
+    down_output = torch.empty((num_groups, m, gate_down_weight.size(1)), device=a.device, dtype=out_dtype)
+    m_grouped_fp8_gemm_nt_masked((down_input, down_input_scale), (gate_down_weight, gate_down_scale), down_output, masked_m,
+                                 expected_m)
+    return down_output

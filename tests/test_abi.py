@@ -83,6 +83,50 @@ def test_argument_validation_rejects_before_touching_the_device():
         _lib.check(_lib.ERR_LAUNCH)
 
 
+def test_moe_entry_points_validate_on_the_host():
+    """The quantisers and the MoE steps refuse bad arguments before any launch (no GPU needed)."""
+    lib = _lib.load()
+    null, fake = ctypes.c_void_p(0), ctypes.c_void_p(4096)
+    assert lib.dlb_fp8_quant_1x128(fake, 0, fake, fake, 4, 100, 100, 1, 1, 1e-10, null) == _lib.ERR_BAD_SHAPE
+    assert lib.dlb_fp8_quant_1x128(fake, 9, fake, fake, 4, 128, 128, 1, 1, 1e-10, null) == _lib.ERR_BAD_DTYPE
+    assert lib.dlb_fp8_quant_128x128(fake, 0, fake, fake, 1, 128, 132, 132, 1e-10, null) == _lib.ERR_BAD_SHAPE
+    assert lib.dlb_fp8_quant_128x128(fake, 0, fake, null, 1, 128, 128, 128, 1e-10, null) == _lib.ERR_NULL_POINTER
+    assert lib.dlb_fp8_quant_128x128(fake, 0, fake, fake, 1, 128, 128, 64, 1e-10, null) == _lib.ERR_BAD_STRIDE
+    assert lib.dlb_fp8_quant_128x128(null, 0, null, null, 0, 128, 128, 128, 1e-10, null) == 0
+    assert lib.dlb_silu_mul(fake, 3, fake, 4, 128, 256, 128, null) == _lib.ERR_BAD_DTYPE
+    assert lib.dlb_silu_mul(fake, 0, fake, 4, 128, 128, 128, null) == _lib.ERR_BAD_STRIDE
+    assert lib.dlb_silu_mul(fake, 0, null, 4, 128, 256, 128, null) == _lib.ERR_NULL_POINTER
+    assert lib.dlb_silu_mul_quant(fake, 0, fake, fake, 4, 200, 400, 2, 1, 1e-10, null) == _lib.ERR_BAD_SHAPE
+    assert lib.dlb_silu_mul_quant(ctypes.c_void_p(4100), 0, fake, fake, 4, 128, 256, 1, 1, 1e-10, null) == _lib.ERR_ALIGNMENT
+    assert lib.dlb_silu_mul_quant_masked(fake, 0, fake, fake, null, 2, 4, 128, 4, 1, 1, null) == _lib.ERR_NULL_POINTER
+    assert lib.dlb_silu_mul_quant_masked(fake, 0, fake, fake, fake, -1, 4, 128, 4, 1, 1, null) == _lib.ERR_BAD_SHAPE
+    assert lib.dlb_silu_mul_quant_masked(fake, 0, fake, fake, fake, 2, 4, 128, 4, -1, 1, null) == _lib.ERR_BAD_STRIDE
+    # ep_scatter: hidden % 128, topk limit, workspace size, index dtypes
+    def scatter(hidden=256, topk=8, experts=4, ws=fake, ws_bytes=1 << 20, topk_dtype=0, x=fake):
+        return lib.dlb_ep_scatter(x, hidden, fake, hidden // 128, 1, fake, topk_dtype, topk, 1, fake, fake, 0, fake, hidden, fake,
+                                  hidden // 128, 1, fake, 512, fake, 0, topk, 1, 16, hidden, topk, experts, ws, ws_bytes, null)
+    assert scatter(hidden=200) == _lib.ERR_BAD_SHAPE
+    assert scatter(topk=65) == _lib.ERR_BAD_SHAPE and '64' in _lib.last_error()
+    assert scatter(experts=5000) == _lib.ERR_BAD_SHAPE
+    assert scatter(topk_dtype=2) == _lib.ERR_BAD_DTYPE
+    assert scatter(ws=null) == _lib.ERR_WORKSPACE and scatter(ws_bytes=8) == _lib.ERR_WORKSPACE
+    assert scatter(x=ctypes.c_void_p(4100)) == _lib.ERR_ALIGNMENT
+    assert scatter(experts=0) == 0
+    need = lib.dlb_ep_scatter_workspace_bytes(8192, 8, 32)
+    assert need == (32 + 2) * 8 + 256 * 32 * 4
+    # ep_gather
+    def gather(hidden=1024, topk=8, in_dtype=0, out=fake):
+        return lib.dlb_ep_gather(fake, in_dtype, hidden, fake, 0, topk, 1, fake, topk, 1, fake, 0, topk, 1, out, 0, hidden, 16,
+                                 hidden, topk, null)
+    assert gather(hidden=1020) == _lib.ERR_BAD_SHAPE
+    assert gather(topk=100) == _lib.ERR_BAD_SHAPE
+    assert gather(in_dtype=5) == _lib.ERR_BAD_DTYPE
+    assert gather(out=null) == _lib.ERR_NULL_POINTER
+    assert lib.dlb_scale_relayout(fake, fake, 8, 4, 4, 4, 1, null) == _lib.ERR_BAD_SHAPE      # rows_pad < rows
+    assert lib.dlb_scale_relayout(fake, null, 8, 4, 8, 4, 1, null) == _lib.ERR_NULL_POINTER
+    assert lib.dlb_scale_relayout(null, null, 0, 0, 0, 1, 1, null) == 0
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, '_lib', None)
     monkeypatch.setenv('DLBLAS_AMD_LIB', str(tmp_path / 'nope.so'))
