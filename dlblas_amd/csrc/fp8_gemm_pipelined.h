@@ -223,28 +223,44 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     const uint32_t dma_chunk = static_cast<uint32_t>(((lane & 7) ^ chunk_swizzle(dma_row)) * 16);
     const uint32_t uK = static_cast<uint32_t>(p.K);
 
+    // Per-lane source offsets of every DMA instruction of a stage, computed once per tile: the K loop then issues
+    // its DMA group without any vector ALU work (32-bit multiplies are quarter rate and, issued right behind the
+    // barrier by every wave at once, kept the matrix pipe waiting).
+    uint32_t a_off[Cfg::A_INST], b_off[Cfg::B_INST], s_off[Cfg::S_INST];
+#pragma unroll
+    for (int j = 0; j < Cfg::A_INST; ++j)
+      a_off[j] = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, a_last)) * uK + dma_chunk;
+#pragma unroll
+    for (int j = 0; j < Cfg::B_INST; ++j)
+      b_off[j] = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, b_last)) * uK + dma_chunk;
+#pragma unroll
+    for (int j = 0; j < Cfg::S_INST; ++j)
+      s_off[j] = static_cast<uint32_t>(min((j * WAVES + wave) * 64 + lane, a_last)) * static_cast<uint32_t>(p.as_sm) * 4u;
+
     auto issue_stage = [&](int kb, int stage) {
       uint8_t* sbase = smem + stage * Cfg::STAGE_BYTES;
       const uint8_t* ag = a_tile + static_cast<int64_t>(kb) * kScaleBlock;
       const uint8_t* bg = b_tile + static_cast<int64_t>(kb) * kScaleBlock;
       const uint8_t* sg = reinterpret_cast<const uint8_t*>(as_tile + static_cast<int64_t>(kb) * p.as_sk);
-      int row0 = dma_row;
-      asm volatile("" : "+v"(row0));  // keeps the per-instruction offsets out of loop-invariant registers
+      // the empty asm keeps each offset a 32-bit register here, so that the load uses the scalar-base + 32-bit
+      // vector-offset form instead of a 64-bit address built outside the loop (two registers per instruction)
 #pragma unroll
       for (int j = 0; j < Cfg::A_INST; ++j) {
-        const uint32_t off = static_cast<uint32_t>(min(row0 + 8 * j * WAVES, a_last)) * uK + dma_chunk;
-        dma_16(ag, off, sbase + (j * WAVES + wave) * 1024);
+        uint32_t o = a_off[j];
+        asm volatile("" : "+v"(o));
+        dma_16(ag, o, sbase + (j * WAVES + wave) * 1024);
       }
 #pragma unroll
       for (int j = 0; j < Cfg::B_INST; ++j) {
-        const uint32_t off = static_cast<uint32_t>(min(row0 + 8 * j * WAVES, b_last)) * uK + dma_chunk;
-        dma_16(bg, off, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
+        uint32_t o = b_off[j];
+        asm volatile("" : "+v"(o));
+        dma_16(bg, o, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
       }
 #pragma unroll
       for (int j = 0; j < Cfg::S_INST; ++j) {
-        const int row = (j * WAVES + wave) * 64 + lane;
-        const uint32_t off = static_cast<uint32_t>(min(row, a_last)) * static_cast<uint32_t>(p.as_sm) * 4u;
-        dma_4(sg, off, sbase + Cfg::A_BYTES + Cfg::B_BYTES + (j * WAVES + wave) * 256);
+        uint32_t o = s_off[j];
+        asm volatile("" : "+v"(o));
+        dma_4(sg, o, sbase + Cfg::A_BYTES + Cfg::B_BYTES + (j * WAVES + wave) * 256);
       }
       // weight scales of the wave's fragments at this K block, one per lane slot
       dma_4(reinterpret_cast<const uint8_t*>(bs_g + kb), bs_off,
