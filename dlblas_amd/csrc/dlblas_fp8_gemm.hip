@@ -493,20 +493,40 @@ int run(const Problem& pr) {
   }
 
   hipError_t e = hipSuccess;
+  // expert-contiguous rows: a device-built list of 256- and 128-row tiles (see contiguous_tile_list_kernel); its
+  // storage sits at the head of the workspace's data region, the re-laid scales behind it
+  size_t ws_used = 0;
+  bool tile_list = false;
+  if (pr.mode == kContiguous && pl.variant == kVarPipe128x256w8 && g_forced_variant < 0 && ar.ws && kblocks > 0) {
+    const int64_t nblk = ceil_div(pr.rows, kScaleBlock);
+    const size_t bytes = (static_cast<size_t>(2 + 2 * nblk) * sizeof(int32_t) + 255) / 256 * 256;
+    if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= pr.ws_bytes) {
+      int32_t* tl = reinterpret_cast<int32_t*>(ar.ws);
+      hipLaunchKernelGGL(contiguous_tile_list_kernel, dim3(1), dim3(256), 0, pr.stream, pr.gidx, static_cast<int>(pr.rows), pr.G, tl,
+                         static_cast<int>(nblk));
+      e = hipGetLastError();
+      if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "tile list launch failed: %s", hipGetErrorString(e));
+      ar.tlist = tl;
+      ar.tlist_cap = static_cast<int>(nblk);
+      ws_used = bytes;
+      tile_list = true;
+    }
+  }
   if (is_pipelined(pl.variant) && pr.as_sk == 1 && pr.as_sm > 1 && ar.ws && kblocks > 1) {
     // row-major activation scales: re-lay them rows-contiguous in the workspace first (a few microseconds) so the
     // GEMM fetches 8 cache lines of scales per K step and tile instead of 256
     const int64_t rows_pad = (pr.rows + 3) / 4 * 4;
     const int64_t need = groups * kblocks * rows_pad * static_cast<int64_t>(sizeof(float));
-    if (static_cast<size_t>(need) + DLB_WS_COUNTER_BYTES <= pr.ws_bytes && rows_pad * kblocks < (1ll << 31)) {
+    if (static_cast<size_t>(need) + ws_used + DLB_WS_COUNTER_BYTES <= pr.ws_bytes && rows_pad * kblocks < (1ll << 31)) {
+      float* relaid = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
       const dim3 tgrid(static_cast<unsigned>(ceil_div(rows_pad, 32)), static_cast<unsigned>(ceil_div(kblocks, 32)),
                        static_cast<unsigned>(pr.mode == kMasked ? groups : 1));
-      hipLaunchKernelGGL(fp8_scale_transpose_kernel, tgrid, dim3(256), 0, pr.stream, pr.a_s, ar.ws, static_cast<int>(pr.rows),
+      hipLaunchKernelGGL(fp8_scale_transpose_kernel, tgrid, dim3(256), 0, pr.stream, pr.a_s, relaid, static_cast<int>(pr.rows),
                          static_cast<int>(kblocks), static_cast<int>(rows_pad), pr.mode == kMasked ? pr.as_sg : 0, pr.as_sm,
                          pr.as_sk);
       e = hipGetLastError();
       if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "scale re-layout launch failed: %s", hipGetErrorString(e));
-      ar.a_s = ar.ws;
+      ar.a_s = relaid;
       ar.as_sm = 1;
       ar.as_sk = rows_pad;
       ar.as_gs = kblocks * rows_pad;
@@ -566,7 +586,17 @@ int run(const Problem& pr) {
         e = launch_pipelined_mode<Pipe128x256>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe256x256)
         e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g, dev, pr.stream);
-      else if (pl.variant == kVarPipe128x256w8)
+      else if (pl.variant == kVarPipe128x256w8 && tile_list) {
+        static std::atomic<unsigned long long> lds_done{0};
+        auto kernel = fp8_gemm_contig_list_kernel<Pipe256x256, Pipe128x256w8>;
+        constexpr int lds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES ? Pipe256x256::LDS_BYTES : Pipe128x256w8::LDS_BYTES;
+        e = ensure_lds(kernel, lds, dev, &lds_done);
+        if (e == hipSuccess) {
+          ar.tiles_n = static_cast<int>(ceil_div(pr.N, 256));
+          hipLaunchKernelGGL(kernel, dim3(cus), dim3(Pipe256x256::NT), lds, pr.stream, ar);  // one resident workgroup per CU
+          e = hipGetLastError();
+        }
+      } else if (pl.variant == kVarPipe128x256w8)
         e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarTile64x128)
         e = launch_tiled_mode<Tile64x128>(pr.mode, ar, g, dev, pr.stream);

@@ -20,7 +20,7 @@ typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
 
 constexpr int kScaleBlock = 128;  // K (and N) extent covered by one scale; also bytes per LDS tile row
 
-enum Mode : int { kDense = 0, kContiguous = 1, kMasked = 2 };
+enum Mode : int { kDense = 0, kContiguous = 1, kMasked = 2, kContigList = 3 };  // kContigList: contiguous, tiles from a device-built list
 
 // Everything a kernel needs; passed by value as the single kernel argument.
 struct Args {
@@ -56,6 +56,8 @@ struct Args {
   int tiles_a;          //   tiles in the wide region (tiles_m x tiles_n_a)
   int tiles_n_a;
   int tiles_n_b;
+  const int32_t* tlist;  // kContigList: [0] = 256-row tiles, [1] = 128-row tiles, then the two lists of 128-row block indices
+  int tlist_cap;         //   entries per list
 };
 
 // D = A_op * B_op^T with A_op [16 x 128] and B_op [16 x 128] e4m3; lane l supplies row (l & 15) of each

@@ -158,7 +158,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
   int walk_base = 0;
 
   for (int vb = vb_first;; vb += gridDim.x) {
-    int g = 0, mt, nt, m_end;
+    int g = 0, mt = 0, nt, m_end, m_first = -1;
     if (MODE == kMasked) {
       int mtiles = 0;
       while (walk_g < p.G) {
@@ -175,6 +175,18 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       mt = local % mtiles;
       nt = local / mtiles;
       m_end = min(max(p.gidx[g], 0), p.M);
+    } else if (MODE == kContigList) {
+      // tiles of this height come from the list the pre-pass built: entry = first 128-row block of the tile.  The
+      // column tiles of one row block are adjacent in the order, so they share the activation tile in L2.
+      const int cnt = p.tlist[BM == 256 ? 0 : 1];
+      const int total = cnt * tiles_n;
+      if (vb >= total) break;
+      const int t = xcd_remap(vb, total);
+      const int li = t / tiles_n;
+      nt = t - li * tiles_n;
+      m_first = p.tlist[2 + (BM == 256 ? 0 : p.tlist_cap) + li] * 128;
+      g = p.gidx[m_first];
+      m_end = min(p.M, m_first + BM);
     } else {
       if (vb >= tiles) break;
       const int t = xcd_remap(vb, tiles);
@@ -192,7 +204,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       }
     }
     g = __builtin_amdgcn_readfirstlane(g);
-    const int m0 = __builtin_amdgcn_readfirstlane(mt * BM);
+    const int m0 = __builtin_amdgcn_readfirstlane(MODE == kContigList ? m_first : mt * BM);
     const int n0 = __builtin_amdgcn_readfirstlane(n_base + nt * BN);
 
     const int64_t esz = p.out_f32 ? 4 : 2;
@@ -527,6 +539,61 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
 // one workgroup per tile, region A first.  The host picks the cut so that the last round of workgroups fills the
 // chip: e.g. 448 tiles of 256 x 256 on 256 CUs leave a quarter of the chip idle in the second round, while 256
 // tiles of 256 x 256 followed by 256 tiles of 256 x 192 cover the same output and keep every CU busy.
+// Expert-contiguous rows: a one-block pre-pass turns m_indices into two tile lists - 256-row tiles for pairs of
+// adjacent 128-row blocks of the same expert, 128-row tiles for what is left of every expert's run - so that most
+// weight tiles are fetched once per expert instead of once per 128 rows.  Blocks whose first index is negative (or
+// not an expert) appear in no list.  list layout: [0] = n256, [1] = n128, [2 ..] 256-row list, [2 + cap ..] 128-row list.
+constexpr int kTileListMaxBlocks = 4096;  // 512 K rows; more rows fall back to uniform 128-row tiles
+
+__global__ void __launch_bounds__(256) contiguous_tile_list_kernel(const int32_t* m_indices, int M, int G, int32_t* tlist,
+                                                                   int cap) {
+  __shared__ int eb[kTileListMaxBlocks];   // expert of every 128-row block, -1 = skip
+  __shared__ int rs[kTileListMaxBlocks];   // first block of the run of equal experts the block belongs to
+  __shared__ int chunk_last[256];
+  __shared__ int n256, n128;
+  const int tid = threadIdx.x;
+  const int nblk = (M + 127) / 128;
+  if (tid == 0) n256 = n128 = 0;
+  for (int b = tid; b < nblk; b += 256) {
+    const int e = m_indices[static_cast<int64_t>(b) * 128];
+    eb[b] = (e >= 0 && e < G) ? e : -1;
+  }
+  __syncthreads();
+  const int chunk = (nblk + 255) / 256;
+  const int b0 = min(nblk, tid * chunk), b1 = min(nblk, b0 + chunk);
+  int last = -1;
+  for (int b = b0; b < b1; ++b) {
+    if (b == 0 || eb[b] != eb[b - 1]) last = b;
+    rs[b] = last;
+  }
+  chunk_last[tid] = last;
+  __syncthreads();
+  int carry = -1;
+  for (int q = 0; q < tid; ++q) carry = max(carry, chunk_last[q]);
+  for (int b = b0; b < b1 && rs[b] < 0; ++b) rs[b] = carry;
+  __syncthreads();
+  for (int b = tid; b < nblk; b += 256) {
+    if (eb[b] < 0 || ((b - rs[b]) & 1)) continue;  // odd position in its run: second half of a 256-row tile
+    if (b + 1 < nblk && eb[b + 1] == eb[b])
+      tlist[2 + atomicAdd(&n256, 1)] = b;
+    else
+      tlist[2 + cap + atomicAdd(&n128, 1)] = b;
+  }
+  __syncthreads();
+  if (tid == 0) tlist[0] = n256, tlist[1] = n128;
+}
+
+template <class CfgA, class CfgB>
+__global__ void __launch_bounds__(CfgA::NT) fp8_gemm_contig_list_kernel(const Args p) {
+  static_assert(CfgA::NT == CfgB::NT && CfgA::BN == CfgB::BN, "both tile heights use the same workgroup shape and width");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // persistent workgroups: tall tiles first, then the short ones continue the round robin where the tall ones ended
+  pipelined_body<CfgA, kContigList>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
+  const int total_a = p.tlist[0] * p.tiles_n;
+  const int first_b = (static_cast<int>(blockIdx.x) + gridDim.x - total_a % gridDim.x) % gridDim.x;
+  pipelined_body<CfgB, kContigList>(p, smem, first_b, 0, p.tiles_n, 0);
+}
+
 template <class CfgA, class CfgB>
 __global__ void __launch_bounds__(CfgA::NT) fp8_gemm_pipelined_mixed_kernel(const Args p) {
   static_assert(CfgA::NT == CfgB::NT && CfgA::BM == CfgB::BM, "both regions use the same workgroup shape and tile height");

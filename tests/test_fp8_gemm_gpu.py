@@ -180,6 +180,35 @@ def test_grouped_contiguous(dev, col_major_scales, out_dtype):
     helpers.tolerance_check(out, ref, 'grouped contiguous')
 
 
+@pytest.mark.parametrize('variant', [None, 'pipe128x256w8', 'tile128x128'])
+def test_grouped_contiguous_run_lengths(dev, variant):
+    """Runs of 1 to 5 blocks of 128 rows, skipped blocks between and inside runs, an expert that owns two separate
+    runs, experts out of order: the library's own choice pairs blocks into 256-row tiles from a list built on the
+    device; forced variants take the uniform 128-row path.  All must agree with the oracle."""
+    print(f'case contiguous run lengths variant={variant}', flush=True)
+    from dlblas_amd import _lib
+    from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_contiguous
+    G, N, K = 5, 520, 384
+    blocks = [3, 3, -1, 0, 0, 0, 0, 0, 2, -1, -1, 4, 4, 4, 3, 1, 1, -1]   # expert of every 128-row block
+    M_sum = 128 * len(blocks)
+    g = helpers.gen(19)
+    a_q, a_s = orc.quant_act_1x128(torch.randn(M_sum, K, generator=g).to(torch.bfloat16))
+    w_q, w_s = _make_grouped_weights(G, N, K, 20)
+    m_indices = torch.tensor(blocks, dtype=torch.int32).repeat_interleave(128)
+    sentinel = 321.0
+    ref = orc.grouped_contiguous_ref(a_q, a_s, w_q, w_s, torch.full((M_sum, N), sentinel), m_indices)
+    out = torch.full((M_sum, N), sentinel, dtype=torch.bfloat16, device=dev)
+    try:
+        _lib.force_variant(variant)
+        m_grouped_fp8_gemm_nt_contiguous((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, m_indices.to(dev))
+        torch.cuda.synchronize()
+    finally:
+        _lib.force_variant(None)
+    skipped = (m_indices < 0)
+    assert torch.all(out.cpu()[skipped] == sentinel), 'a skipped block was written'
+    helpers.tolerance_check(out, ref, f'contiguous run lengths {variant}')
+
+
 def test_grouped_masked(dev):
     print('case masked', flush=True)
     from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
