@@ -86,9 +86,10 @@ enum Knob : int {
   kKnobSkinnyNFrags,
   kKnobGroupM,
   kKnobSkinnyDma,  // 0 / 1: DMA-staged decode kernel where possible, 2: register-load decode kernel
+  kKnobEpilogue,   // 0 / 1: bf16 output of the pipelined kernels goes through LDS where it can, 2: straight from registers
   kKnobCount
 };
-thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0};
+thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0};
 
 enum Variant : int {
   kVarExact = 0,
@@ -487,6 +488,7 @@ int run(const Problem& pr) {
   ar.out_f32 = pr.out_dtype == DLB_OUT_F32;
   const size_t esz = ar.out_f32 ? 4 : 2;
   ar.vec_store = (pr.N % 4 == 0) && !misaligned(pr.c, 4 * esz);
+  ar.c_vec16 = !ar.out_f32 && pr.N % 8 == 0 && !misaligned(pr.c, 16) && g_knob[kKnobEpilogue] != 2;
   if (pr.ws && pr.ws_bytes >= DLB_WS_COUNTER_BYTES) {
     ar.ctr = static_cast<uint32_t*>(pr.ws);
     ar.ws = reinterpret_cast<float*>(static_cast<char*>(pr.ws) + DLB_WS_COUNTER_BYTES);

@@ -52,6 +52,7 @@ struct Args {
   int group_m;          // m-tiles per L2 swizzle group
   int out_f32;
   int vec_store;        // rows of c are aligned for 4-element vector stores
+  int c_vec16;          // bf16 c whose rows are 16-byte aligned (N % 8 == 0): the LDS-transposed epilogue applies
   int n_split;          // mixed-width launch: first column of the narrow-tile region
   int tiles_a;          //   tiles in the wide region (tiles_m x tiles_n_a)
   int tiles_n_a;

@@ -508,6 +508,42 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     }
 
     // epilogue: lane holds c[m0 + wm0 + 32 mi + (lane & 31)][n0 + wn0 + 32 ni + 8 u + 4 (lane >> 5) + 0..3], u = 0..3
+    if (p.c_vec16) {
+      // bf16 through LDS: stored straight from the accumulator layout every instruction would touch 32 rows with
+      // 16 bytes each, partial sectors that the L2 has to merge.  Each wave parks its 64-row tile in its own slice of
+      // the (now idle) ring, rows rotated by their index to spread the banks, and reads it back row-wise: a store
+      // instruction then writes whole rows, 16 bytes per lane.
+      constexpr int kRowBytes = NF * 32 * 2;
+      constexpr int kCpr = kRowBytes / 16;   // 16-byte chunks per row
+      constexpr int kRpi = 64 / kCpr;        // rows per store instruction
+      static_assert(MF * 32 * kRowBytes * WAVES <= Cfg::LDS_BYTES, "the staging slices fit in the ring");
+      __syncthreads();  // every wave is done reading the ring
+      uint8_t* st = smem + wave * (MF * 32 * kRowBytes);
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) {
+        const int row = mi * 32 + l32;
+#pragma unroll
+        for (int ni = 0; ni < NF; ++ni)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const v4f v = {acc[mi][ni][4 * u], acc[mi][ni][4 * u + 1], acc[mi][ni][4 * u + 2], acc[mi][ni][4 * u + 3]};
+            const int chunk = (ni * 4 + u + row) % kCpr;
+            *reinterpret_cast<v4bf*>(st + row * kRowBytes + chunk * 16 + h * 8) = __builtin_convertvector(v, v4bf);
+          }
+      }
+      // a wave reads only what it wrote: no barrier, the LDS counter orders the two
+      const int r_in = lane / kCpr, ch = lane % kCpr;
+      __bf16* c_tile = reinterpret_cast<__bf16*>(c_base) + static_cast<int64_t>(m0 + wm0) * p.N + n0 + wn0;
+#pragma unroll 4
+      for (int r0 = 0; r0 < MF * 32; r0 += kRpi) {
+        const int row = r0 + r_in;
+        if (lane >= kRpi * kCpr || row >= MF * 32) continue;
+        const v4i v = *reinterpret_cast<const v4i*>(st + row * kRowBytes + ((ch + row) % kCpr) * 16);
+        if (m0 + wm0 + row < m_end && n0 + wn0 + ch * 8 < p.N)
+          *reinterpret_cast<v4i*>(c_tile + static_cast<int64_t>(row) * p.N + ch * 8) = v;
+      }
+      continue;
+    }
 #pragma unroll
     for (int mi = 0; mi < MF; ++mi) {
       const int m = m0 + wm0 + mi * 32 + l32;

@@ -84,6 +84,24 @@ def test_split_k_two_pass(dev, M, N, K, variant, splitk, out_dtype):
     assert torch.equal(out, again)
 
 
+@pytest.mark.parametrize('variant', ['pipe256x256', 'pipe128x256w8', 'pipe256mix', 'pipe256x128'])
+@pytest.mark.parametrize('M,N,K', [(200, 392, 2048), (513, 1032, 256)])
+def test_epilogue_through_lds_equals_direct_stores(dev, variant, M, N, K):
+    """bf16 results of the pipelined kernels leave through an LDS transpose (whole rows per store instruction) or, by
+    knob, straight from the accumulator registers: the same fp32 values, the same rounding, the same bits."""
+    from dlblas_amd import _lib
+    print(f'case epilogue variant={variant} M={M} N={N} K={K}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=23)
+    try:
+        _lib.tune('epilogue', 2)
+        direct = _run_dense(dev, a_q, a_s, b_q, b_s, variant=variant)
+    finally:
+        _lib.tune('epilogue', 0)
+    staged = _run_dense(dev, a_q, a_s, b_q, b_s, variant=variant)
+    assert torch.equal(direct, staged)
+    helpers.tolerance_check(staged, orc.dequant_ref(a_q, a_s, b_q, b_s), f'epilogue {variant}')
+
+
 def test_dense_f32_reference_test_construction(dev):
     """The reference's own test: randn e4m3 operands, randn (signed) scales, fp32 out, atol 1e-1
     (tests/kernels/test_fp8_gemm.py:8-31,70-72)."""
