@@ -375,6 +375,8 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
     // K is split over the waves of a workgroup only.  Pick the wave count so that every wave has two or so K
     // blocks and the unroll so that a wave issues all of its loads before its first MFMA.
     int waves = kblocks >= 8 ? 8 : 4;
+    // 128 activation rows: only four waves' staging areas (10 blocks of 2 KB per wave and K block) fit in LDS
+    if (v == kVarSkinny128) waves = 4;
     if (g_knob[kKnobSkinnyWaves] > 0) waves = g_knob[kKnobSkinnyWaves];
     const int per_wave = static_cast<int>(ceil_div(kblocks, waves));
     // measured on MI355X: one K block in flight per wave is as good as more once eight waves share a row block
