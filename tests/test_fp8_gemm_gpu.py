@@ -102,6 +102,36 @@ def test_epilogue_through_lds_equals_direct_stores(dev, variant, M, N, K):
     helpers.tolerance_check(staged, orc.dequant_ref(a_q, a_s, b_q, b_s), f'epilogue {variant}')
 
 
+def _random_shapes(n, seed):
+    import random
+    rng = random.Random(seed)
+    shapes = []
+    for _ in range(n):
+        kind = rng.random()
+        M = rng.choice([1, 2, 15, 16, 17, 31, 33, 64, 65, 127, 128, 129, 255, 257, 300, 511, 640])
+        N = rng.choice([1, 7, 8, 24, 128, 130, 192, 200, 256, 264, 392, 520, 776, 1032])
+        if kind < 0.6:
+            K = 128 * rng.randint(1, 18)
+        elif kind < 0.85:
+            K = 16 * rng.randint(1, 60)
+        else:
+            K = rng.randint(1, 300)
+        shapes.append((M, N, K))
+    return shapes
+
+
+@pytest.mark.parametrize('M,N,K', _random_shapes(40, 2024))
+def test_dense_random_shapes_take_the_library_choice(dev, M, N, K):
+    """Seeded random shapes across every branch of the shape heuristic (decode, split-K, pipelined, mixed, tiled with
+    K tails, exact), bf16 and fp32 alternating."""
+    out_dtype = torch.float32 if (M + N + K) % 2 else torch.bfloat16
+    print(f'case random M={M} N={N} K={K} {out_dtype}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=M * 7 + N * 3 + K)
+    out = _run_dense(dev, a_q, a_s, b_q, b_s, dtype=out_dtype)
+    assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
+    helpers.tolerance_check(out, orc.dequant_ref(a_q, a_s, b_q, b_s), f'random {M}x{N}x{K}')
+
+
 def test_dense_f32_reference_test_construction(dev):
     """The reference's own test: randn e4m3 operands, randn (signed) scales, fp32 out, atol 1e-1
     (tests/kernels/test_fp8_gemm.py:8-31,70-72)."""
