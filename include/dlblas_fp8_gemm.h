@@ -19,7 +19,8 @@
  *   - `workspace` is caller-owned device memory of at least dlb_fp8_gemm_workspace_bytes()
  *     bytes, 16-byte aligned.  Its first DLB_WS_COUNTER_BYTES bytes are reserved (no kernel
  *     of this version reads or writes them); the rest is scratch that a call overwrites:
- *     re-laid activation scales, fp32 partial sums of the split-K path.  Nothing in it has
+ *     re-laid activation scales, fp32 partial sums of the split-K path, the tile list of the
+ *     expert-contiguous path.  Nothing in it has
  *     to survive between calls, so one buffer serves any number of calls that do not overlap
  *     in time.  Two calls that may run concurrently (different streams) need separate
  *     workspaces.
