@@ -278,6 +278,32 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       dma_4(reinterpret_cast<const uint8_t*>(bs_g + kb), bs_off,
             sbase + Cfg::A_BYTES + Cfg::B_BYTES + Cfg::S_BYTES + wave * 256);
     };
+    // The same group, one instruction at a time (i = 0 .. LOADS_PER_STAGE - 1, compile-time): the in-place K loop
+    // spreads a stage's DMA over several tile slots instead of issuing it in one burst behind the barrier, where
+    // the eight waves' 80 instructions queue up in front of the texture path and keep the waves from their MFMAs.
+    auto issue_one = [&](auto idx, int kb, int stage) __attribute__((always_inline)) {
+      constexpr int i = decltype(idx)::value;
+      uint8_t* sbase = smem + stage * Cfg::STAGE_BYTES;
+      if constexpr (i < Cfg::A_INST) {
+        uint32_t o = a_off[i];
+        asm volatile("" : "+v"(o));
+        dma_16(a_tile + static_cast<int64_t>(kb) * kScaleBlock, o, sbase + (i * WAVES + wave) * 1024);
+      } else if constexpr (i < Cfg::A_INST + Cfg::B_INST) {
+        constexpr int j = i - Cfg::A_INST;
+        uint32_t o = b_off[j];
+        asm volatile("" : "+v"(o));
+        dma_16(b_tile + static_cast<int64_t>(kb) * kScaleBlock, o, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
+      } else if constexpr (i < Cfg::A_INST + Cfg::B_INST + Cfg::S_INST) {
+        constexpr int j = i - Cfg::A_INST - Cfg::B_INST;
+        uint32_t o = s_off[j];
+        asm volatile("" : "+v"(o));
+        dma_4(reinterpret_cast<const uint8_t*>(as_tile + static_cast<int64_t>(kb) * p.as_sk), o,
+              sbase + Cfg::A_BYTES + Cfg::B_BYTES + (j * WAVES + wave) * 256);
+      } else {
+        dma_4(reinterpret_cast<const uint8_t*>(bs_g + kb), bs_off,
+              sbase + Cfg::A_BYTES + Cfg::B_BYTES + Cfg::S_BYTES + wave * 256);
+      }
+    };
 
     v16f acc[MF][NF];
 #pragma unroll
@@ -435,6 +461,22 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       const int cur_base = stage * Cfg::STAGE_BYTES;
       const int nxt_base = next_stage * Cfg::STAGE_BYTES;
       float sc_next[MF][NS];
+      // DMA slots: the group that refills this step's stage starts at the barrier slot kP and is spread over kSlots
+      // tile slots, wrapping into the next step (whose slots t < kP therefore finish the PREVIOUS step's group)
+      constexpr int kP = (S - 1) * H;
+      constexpr int kSlots = T >= 8 ? 5 : (T >= 4 ? 3 : 1);  // measured: 3 to 5 of 8 slots are equally good, 6 and 7 leave the loads too little time
+      constexpr int L = Cfg::LOADS_PER_STAGE;
+      const int prev_stage = stage == 0 ? STAGES - 1 : stage - 1;
+      const int kb_new = min(kb + STAGES, nk - 1), kb_prev = min(kb + STAGES - 1, nk - 1);
+      auto issue_slot = [&](auto qtag, int kbx, int stg) __attribute__((always_inline)) {
+        constexpr int q = decltype(qtag)::value;
+        constexpr int i0 = q * L / kSlots, i1 = (q + 1) * L / kSlots;
+        if constexpr (i0 + 0 < i1) issue_one(std::integral_constant<int, i0 + 0>{}, kbx, stg);
+        if constexpr (i0 + 1 < i1) issue_one(std::integral_constant<int, i0 + 1>{}, kbx, stg);
+        if constexpr (i0 + 2 < i1) issue_one(std::integral_constant<int, i0 + 2>{}, kbx, stg);
+        if constexpr (i0 + 3 < i1) issue_one(std::integral_constant<int, i0 + 3>{}, kbx, stg);
+        static_assert(i1 - i0 <= 4, "at most four DMA instructions per slot");
+      };
 #pragma unroll
       for (int t = 0; t < T; ++t) {
         const int si = t / H, hi = t % H;
@@ -444,7 +486,22 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
             wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
             lds_barrier();
           }
-          if (!(DLB_EXP & 1)) issue_stage(min(kb + STAGES, nk - 1), stage);
+        }
+        if (!(DLB_EXP & 1)) {
+          if (t >= kP) {
+            if (t - kP < kSlots) {
+              if (t - kP == 0) issue_slot(std::integral_constant<int, 0>{}, kb_new, stage);
+              if (t - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_new, stage);
+              if (t - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_new, stage);
+              if (t - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_new, stage);
+              if (t - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_new, stage);
+            }
+          } else if (t + T - kP < kSlots) {
+            if (t + T - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_prev, prev_stage);
+            if (t + T - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_prev, prev_stage);
+            if (t + T - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_prev, prev_stage);
+            if (t + T - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_prev, prev_stage);
+          }
         }
         // The scheduling fences pin the order MFMA pair -> reloads -> scale FMAs; without them the compiler
         // hoists the reloads above the MFMAs into fresh registers and the kernel spills.
