@@ -133,7 +133,7 @@ def force_variant(name_or_id) -> None:
     check(lib.dlb_fp8_gemm_force_variant(int(name_or_id)))
 
 
-KNOBS = {'splitk': 0, 'skinny_waves': 1, 'skinny_unroll': 2, 'skinny_nfrags': 3, 'group_m': 4, 'skinny_dma': 5, 'epilogue': 6}
+KNOBS = {'splitk': 0, 'skinny_waves': 1, 'skinny_unroll': 2, 'skinny_nfrags': 3, 'group_m': 4, 'skinny_dma': 5, 'epilogue': 6, 'skinny_bn': 7}
 
 
 def tune(knob: str, value) -> None:

@@ -87,9 +87,10 @@ enum Knob : int {
   kKnobGroupM,
   kKnobSkinnyDma,  // 0 / 1: DMA-staged decode kernel where possible, 2: register-load decode kernel
   kKnobEpilogue,   // 0 / 1: bf16 output of the pipelined kernels goes through LDS where it can, 2: straight from registers
+  kKnobSkinnyBn,   // columns per workgroup of the DMA-staged decode kernels (0 = heuristic)
   kKnobCount
 };
-thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0};
+thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0, 0};
 
 enum Variant : int {
   kVarExact = 0,
@@ -186,7 +187,8 @@ hipError_t launch_skinny_cfg(const Args& args, int dev, hipStream_t stream) {
     auto kernel = fp8_gemm_skinny_dma_kernel<Cfg>;
     hipError_t e = ensure_lds(kernel, Cfg::DMA_LDS_BYTES, dev, &lds_done_dma);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kernel, dim3(args.tiles_n), dim3(Cfg::NT), Cfg::DMA_LDS_BYTES, stream, args);
+    const unsigned grid = static_cast<unsigned>(ceil_div(args.N, args.sk_bn));  // its own column split, see pick_skinny_bn
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NT), Cfg::DMA_LDS_BYTES, stream, args);
     return hipGetLastError();
   }
   auto kernel = ktail ? fp8_gemm_skinny_kernel<Cfg, true> : fp8_gemm_skinny_kernel<Cfg, false>;
@@ -282,6 +284,7 @@ struct Plan {
   int bm, bn;
   int splitk;
   int sk_waves, sk_unroll, sk_nfrags;  // skinny kernel shape
+  int sk_bn;                           // columns per workgroup of its DMA-staged form
 };
 
 void tile_dims(int variant, int* bm, int* bn) {
@@ -333,8 +336,25 @@ int clamp_splitk(int want, int64_t M, int64_t N, int kblocks, size_t avail) {
   return s < 1 ? 1 : s;
 }
 
+// Output columns per workgroup of the DMA-staged decode kernels.  A CU streams weights at a rate of its own (about
+// 1 / 256 of what the chip reaches), so the launch takes as long as its busiest CU: the split that gives every CU
+// the same number of weight rows wins, e.g. 28 columns for N = 7168 on 256 CUs (256 workgroups) instead of 32 (224),
+// or 12 for N = 2112 (176 workgroups) instead of 16 (132).  Every workgroup also reads all activation rows (from the
+// L2, cheaper per row); several rounds of workgroups cost in proportion.  Multiples of 4 keep a lane's four output
+// columns inside one workgroup and one 128-column scale block.
+int pick_skinny_bn(int64_t N, int act_rows, int cus) {
+  int best = 16;
+  double best_cost = 0.0;
+  for (int bn = 4; bn <= 32; bn += 4) {
+    const int64_t wgs = ceil_div(N, bn);
+    const double cost = static_cast<double>(ceil_div(wgs, cus)) * (bn + 0.4 * act_rows);
+    if (bn == 4 || cost < best_cost - 1e-9) best = bn, best_cost = cost;
+  }
+  return best;
+}
+
 Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes) {
-  Plan pl{kVarTile128x128, 128, 128, 1, 4, 4, 1};
+  Plan pl{kVarTile128x128, 128, 128, 1, 4, 4, 1, 16};
   const int kblocks = static_cast<int>(ceil_div(K, kScaleBlock));
   int v = g_forced_variant;
   if (v < 0) {
@@ -386,6 +406,12 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
     int nfrags = ceil_div(N, 32) * 4 >= 3 * cus ? 2 : 1;
     if (g_knob[kKnobSkinnyNFrags] > 0) nfrags = g_knob[kKnobSkinnyNFrags];
     pl.sk_waves = waves, pl.sk_unroll = unroll, pl.sk_nfrags = nfrags >= 2 ? 2 : 1;
+    pl.sk_bn = 16 * pl.sk_nfrags;
+    if (g_knob[kKnobSkinnyNFrags] <= 0 && K % kScaleBlock == 0) {
+      pl.sk_bn = g_knob[kKnobSkinnyBn] > 0 ? g_knob[kKnobSkinnyBn] : pick_skinny_bn(N, skinny_rows(v), cus);
+      if (pl.sk_bn % 4 != 0 || pl.sk_bn < 4 || pl.sk_bn > 32) pl.sk_bn = 16 * pl.sk_nfrags;
+      pl.sk_nfrags = pl.sk_bn > 16 ? 2 : 1;
+    }
     pl.bn = 16 * pl.sk_nfrags;
   } else {
     // few tiles and a long K: split K over workgroups (partial sums in the workspace, second pass adds them)
@@ -483,6 +509,7 @@ int run(const Problem& pr) {
   ar.bs_gs = static_cast<int64_t>(ar.nblocks) * kblocks;
   ar.tiles_m = static_cast<int>(ceil_div(pr.rows, pl.bm));
   ar.tiles_n = static_cast<int>(ceil_div(pr.N, pl.bn));
+  ar.sk_bn = pl.sk_bn;
   ar.splitk = pl.splitk;
   ar.kb_per_split = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, pl.splitk));
   ar.splitk = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, ar.kb_per_split));  // no empty splits

@@ -47,6 +47,7 @@ struct Args {
   int nblocks;          // ceil(N / 128)
   int tiles_m;
   int tiles_n;
+  int sk_bn;            // decode kernels with DMA staging: output columns per workgroup (multiple of 4, <= 16 NFS)
   int splitk;
   int kb_per_split;
   int group_m;          // m-tiles per L2 swizzle group

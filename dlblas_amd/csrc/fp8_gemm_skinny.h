@@ -172,7 +172,11 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l16 = lane & 15;
   const int q = lane >> 4;
-  const int n0 = blockIdx.x * Cfg::BN;
+  // the workgroup owns columns [n0, n0 + cols): p.sk_bn of them (a multiple of 4, at most 16 NFS, chosen on the
+  // host so that the workgroups cover the CUs evenly), fewer at the end of N; fragment rows past them re-read the
+  // last owned row and their results are dropped
+  const int n0 = blockIdx.x * p.sk_bn;
+  const int cols = min(p.sk_bn, p.N - n0);
   const int nk = p.kblocks;
   uint8_t* stage = smem + wave * WAVE_BYTES;
 
@@ -185,7 +189,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
     const uint32_t chunk = static_cast<uint32_t>(((lane & 7) ^ skinny_swizzle(row)) * 16);
 #pragma unroll
     for (int ni = 0; ni < NFS; ++ni)
-      w_off[ni][j] = static_cast<uint32_t>(min(ni * 16 + row, p.N - 1 - n0)) * static_cast<uint32_t>(p.K) + chunk;
+      w_off[ni][j] = static_cast<uint32_t>(min(ni * 16 + row, cols - 1)) * static_cast<uint32_t>(p.K) + chunk;
 #pragma unroll
     for (int mi = 0; mi < MF; ++mi)
       x_off[mi][j] = static_cast<uint32_t>(min(mi * 16 + row, p.M - 1)) * static_cast<uint32_t>(p.K) + chunk;
@@ -196,10 +200,12 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
   const int rd0 = l16 * 128 + (((2 * q) ^ sw) << 4);
   const int rd1 = l16 * 128 + (((2 * q + 1) ^ sw) << 4);
 
+  // weight scales per lane: n0 is any multiple of 4, so a fragment can straddle two 128-column scale blocks, the four
+  // columns of a lane (n0 + 16 ni + 4 q ..) cannot
   const float* bs_row[NFS];
 #pragma unroll
   for (int ni = 0; ni < NFS; ++ni)
-    bs_row[ni] = p.b_s + static_cast<int64_t>(min((n0 + ni * 16) / kScaleBlock, p.nblocks - 1)) * nk;
+    bs_row[ni] = p.b_s + static_cast<int64_t>(min((n0 + ni * 16 + q * 4) / kScaleBlock, p.nblocks - 1)) * nk;
   const float* as_row[MF];
 #pragma unroll
   for (int mi = 0; mi < MF; ++mi) as_row[mi] = p.a_s + static_cast<int64_t>(min(mi * 16 + l16, p.M - 1)) * p.as_sm;
@@ -283,12 +289,12 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
     for (int w = 1; w < WAVES; ++w) sum += red[w][j][lane];
     const int m = mi * 16 + l16;
     const int n = n0 + ni * 16 + q * 4;
-    if (m >= p.M) continue;
+    if (m >= p.M || n >= n0 + cols) continue;
     char* c_row = static_cast<char*>(p.c) + static_cast<int64_t>(m) * p.N * esz;
     if (p.out_f32)
-      store_row4<true>(c_row, n, sum, p.N - n, p.vec_store);
+      store_row4<true>(c_row, n, sum, n0 + cols - n, p.vec_store);
     else
-      store_row4<false>(c_row, n, sum, p.N - n, p.vec_store);
+      store_row4<false>(c_row, n, sum, n0 + cols - n, p.vec_store);
   }
 }
 

@@ -196,6 +196,7 @@ int dlb_fp8_gemm_force_variant(int variant);
  *   DLB_KNOB_GROUP_M        m-tiles per L2 swizzle group of the tiled kernels
  *   DLB_KNOB_SKINNY_DMA     2 = decode kernels load operands through registers instead of the LDS DMA path
  *   DLB_KNOB_EPILOGUE       2 = the pipelined kernels store bf16 results straight from registers (no LDS transpose)
+ *   DLB_KNOB_SKINNY_BN      output columns per workgroup of the DMA-staged decode kernels (multiple of 4, at most 32)
  */
 #define DLB_KNOB_SPLITK 0
 #define DLB_KNOB_SKINNY_WAVES 1
@@ -204,6 +205,7 @@ int dlb_fp8_gemm_force_variant(int variant);
 #define DLB_KNOB_GROUP_M 4
 #define DLB_KNOB_SKINNY_DMA 5
 #define DLB_KNOB_EPILOGUE 6
+#define DLB_KNOB_SKINNY_BN 7
 int dlb_fp8_gemm_tune(int knob, int value);
 
 /* Name of kernel variant `variant`, or NULL beyond the last one. */
