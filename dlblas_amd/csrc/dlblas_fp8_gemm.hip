@@ -106,11 +106,13 @@ enum Variant : int {
   kVarPipe256x256,
   kVarPipe128x256w8,
   kVarPipe256mix,
+  kVarPipe128x128,
+  kVarPipe128x64,
   kVarCount
 };
 
 const char* const kVariantNames[kVarCount] = {
-    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "skinny64", "skinny128", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8", "pipe256mix",
+    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "skinny64", "skinny128", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8", "pipe256mix", "pipe128x128", "pipe128x64",
 };
 
 typedef TileCfg<128, 128, 2, 2> Tile128x128;
@@ -121,6 +123,9 @@ typedef PipeCfg<2, 2, 2, 4, 3, 2, true> Pipe128x256;  // 4 waves, wave tile 64 x
 typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256;  // 8 waves, wave tile 64 x 128
 typedef PipeCfg<4, 2, 2, 3, 2, 2> Pipe256x192;  // narrow tiles of the mixed-width launch
 typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
+// small tiles for problems with few of the large ones (M of a few hundred, or a narrow N): 4 waves, deep rings
+typedef PipeCfg<2, 2, 2, 2, 4, 2, true> Pipe128x128;  // wave tile 64 x 64, 4 stages of 34 KB
+typedef PipeCfg<2, 2, 2, 1, 5, 2, true> Pipe128x64;   // wave tile 64 x 32, 5 stages of 26 KB
 
 // Raise a kernel's dynamic LDS limit once per (kernel, device).
 template <class Kernel>
@@ -318,6 +323,9 @@ void tile_dims(int variant, int* bm, int* bn) {
     case kVarPipe256mix:
       *bm = 256, *bn = 256;
       break;
+    case kVarPipe128x64:
+      *bm = 128, *bn = 64;
+      break;
     default:
       *bm = 128, *bn = 128;
   }
@@ -325,7 +333,7 @@ void tile_dims(int variant, int* bm, int* bn) {
 
 bool is_skinny(int v) { return v >= kVarSkinny16 && v <= kVarSkinny128; }
 int skinny_rows(int v) { return 16 << (v - kVarSkinny16); }
-bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe256mix; }
+bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe128x64; }
 
 // Split count no larger than `want` whose slices hold at least two K blocks and whose fp32 partial matrices fit.
 int clamp_splitk(int want, int64_t M, int64_t N, int kblocks, size_t avail) {
@@ -353,9 +361,41 @@ int pick_skinny_bn(int64_t N, int act_rows, int cus) {
   return best;
 }
 
+// Dense problems between decode and prefill (a few hundred rows, or more rows against a narrow weight matrix): too
+// few 256 x 256 tiles to fill the chip, and weight rows that come from HBM because only one or two row tiles use
+// them.  There a K step of a DMA-ring kernel lasts about (latency of HBM under load) / (stages in flight), whatever
+// the tile size, so the estimate below is: launches + rounds of workgroups x (fixed part of a tile + K steps x time
+// per step) + the second pass when K is split.  Constants measured on MI355X (microseconds; bytes per microsecond).
+struct MidChoice {
+  int variant, splitk;
+  double us;
+};
+
+MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_avail) {
+  struct Cand { int variant, bm, bn; double step_us; };
+  static const Cand cands[] = {{kVarPipe128x256w8, 128, 256, 0.85}, {kVarPipe128x128, 128, 128, 0.65}, {kVarPipe128x64, 128, 64, 0.50}};
+  const double launch = 2.6, relayout = 2.3, tile_fixed = 2.5, second_pass = 2.5, ws_rate = 2.5e6;
+  MidChoice best{kVarPipe128x256w8, 1, 1e30};
+  const double out_bytes = static_cast<double>(M) * N * sizeof(float);
+  for (const Cand& c : cands) {
+    for (int want : {1, 2, 3, 4, 6, 8}) {
+      if (want > 1 && (kblocks / want < 4 || out_bytes * want > static_cast<double>(ws_avail))) continue;
+      const int per = static_cast<int>(ceil_div(kblocks, want));
+      const int sk = static_cast<int>(ceil_div(kblocks, per));
+      const int64_t units = ceil_div(M, c.bm) * ceil_div(N, c.bn) * sk;
+      double us = launch + relayout + static_cast<double>(ceil_div(units, cus)) * (tile_fixed + per * c.step_us);
+      if (sk > 1) us += second_pass + (2.0 * sk + 0.5) * out_bytes / ws_rate;  // partial sums written, read back, result written
+      if (us < best.us) best = MidChoice{c.variant, sk, us};
+    }
+  }
+  return best;
+}
+
 Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes) {
   Plan pl{kVarTile128x128, 128, 128, 1, 4, 4, 1, 16};
   const int kblocks = static_cast<int>(ceil_div(K, kScaleBlock));
+  const size_t ws_avail = ws_bytes > DLB_WS_COUNTER_BYTES ? ws_bytes - DLB_WS_COUNTER_BYTES : 0;
+  int mid_splitk = 0;  // K slices chosen together with a DMA-ring variant
   int v = g_forced_variant;
   if (v < 0) {
     const bool whole_blocks = K > 0 && K % kScaleBlock == 0;
@@ -368,10 +408,23 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
       // re-read the whole activation matrix from L2; K split over workgroups in two passes is twice as fast there
       // (measured at M = 128: 2112 x 7168 44 -> 22 us, 4096 x 7168 45 -> 23 us; 7168 x 2048 stays: 16 vs 19 us)
       if (M > 64 && kblocks >= 32 && ceil_div(N, 128) * 2 <= cus) v = kVarTile128x128;
+      if (M > 64 && whole_blocks) {
+        // 65 .. 128 rows: the streaming kernel's cost is its workgroups each reading all activation rows from the L2
+        // (about 6.5 TB/s over the chip); a K-split tile kernel wins when the weight matrix is narrow and K long
+        const int bn = pick_skinny_bn(N, 128, cus);
+        const double stream_us = 2.6 + static_cast<double>(ceil_div(N, bn)) * M * K / 6.5e6;
+        const MidChoice mid = pick_mid_plan(M, N, kblocks, cus, ws_avail);
+        if (mid.us < stream_us) v = mid.variant, mid_splitk = mid.splitk;
+        else v = kVarSkinny128;
+      }
     } else if (whole_blocks && mode == kDense) {
       const int64_t t256 = ceil_div(M, 256) * ceil_div(N, 256);
-      const int64_t t128 = ceil_div(M, 128) * ceil_div(N, 256);
-      v = t256 * 2 >= cus ? kVarPipe256mix : (t128 * 4 >= cus ? kVarPipe128x256w8 : kVarTile128x128);
+      if (t256 * 2 >= cus) {
+        v = kVarPipe256mix;
+      } else {
+        const MidChoice mid = pick_mid_plan(M, N, kblocks, cus, ws_avail);
+        v = mid.variant, mid_splitk = mid.splitk;
+      }
     } else if (whole_blocks) {
       v = kVarPipe128x256w8;  // grouped: 128-row tiles never straddle two experts / waste at most 127 masked rows
     } else {
@@ -387,6 +440,7 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
   if (v == kVarExact && mode != kDense) v = kVarTile128x128;
   pl.variant = v;
   tile_dims(v, &pl.bm, &pl.bn);
+  if (mode == kDense && is_pipelined(v) && mid_splitk > 1) pl.splitk = mid_splitk;
   if (mode != kDense || v == kVarExact || is_pipelined(v) || (kblocks < 2 && !is_skinny(v))) return pl;
 
   const int64_t tiles_n = ceil_div(N, pl.bn);
@@ -395,8 +449,6 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
     // K is split over the waves of a workgroup only.  Pick the wave count so that every wave has two or so K
     // blocks and the unroll so that a wave issues all of its loads before its first MFMA.
     int waves = kblocks >= 8 ? 8 : 4;
-    // 128 activation rows: only four waves' staging areas (10 blocks of 2 KB per wave and K block) fit in LDS
-    if (v == kVarSkinny128) waves = 4;
     if (g_knob[kKnobSkinnyWaves] > 0) waves = g_knob[kKnobSkinnyWaves];
     const int per_wave = static_cast<int>(ceil_div(kblocks, waves));
     // measured on MI355X: one K block in flight per wave is as good as more once eight waves share a row block
@@ -480,7 +532,7 @@ int run(const Problem& pr) {
 
   Plan pl = make_plan(pr.mode, pr.rows, pr.N, pr.K, cus, pr.ws ? pr.ws_bytes : 0);
   if (g_knob[kKnobSplitK] > 0 && pr.mode == kDense && pl.variant != kVarExact && !is_skinny(pl.variant) &&
-      !is_pipelined(pl.variant))
+      pl.variant != kVarPipe256mix)
     pl.splitk = clamp_splitk(g_knob[kKnobSplitK], pr.rows, pr.N, static_cast<int>(kblocks) * 2,
                              pr.ws && pr.ws_bytes > DLB_WS_COUNTER_BYTES ? pr.ws_bytes - DLB_WS_COUNTER_BYTES : 0);
   if (pr.ws && misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
@@ -561,7 +613,19 @@ int run(const Problem& pr) {
       ar.as_sm = 1;
       ar.as_sk = rows_pad;
       ar.as_gs = kblocks * rows_pad;
+      ws_used += (static_cast<size_t>(need) + 255) / 256 * 256;
     }
+  }
+  if (ar.splitk > 1 && is_pipelined(pl.variant)) {
+    // the partial matrices of the K slices follow whatever else lives in the workspace; fewer slices if they do not fit
+    const size_t avail = pr.ws_bytes - DLB_WS_COUNTER_BYTES - ws_used;
+    const size_t per_slice = static_cast<size_t>(pr.rows) * pr.N * sizeof(float);
+    if (per_slice * ar.splitk > avail) {
+      const int s = per_slice > 0 && avail / per_slice >= 1 ? static_cast<int>(avail / per_slice) : 1;
+      ar.kb_per_split = static_cast<int>(ceil_div(kblocks, s));
+      ar.splitk = static_cast<int>(ceil_div(kblocks, ar.kb_per_split));
+    }
+    ar.ws = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
   }
   const int64_t tiles = static_cast<int64_t>(ar.tiles_m) * ar.tiles_n * ar.splitk;
   switch (pl.variant) {
@@ -629,6 +693,10 @@ int run(const Problem& pr) {
         }
       } else if (pl.variant == kVarPipe128x256w8)
         e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarPipe128x128)
+        e = launch_pipelined_mode<Pipe128x128>(pr.mode, ar, g, dev, pr.stream);
+      else if (pl.variant == kVarPipe128x64)
+        e = launch_pipelined_mode<Pipe128x64>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarTile64x128)
         e = launch_tiled_mode<Tile64x128>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarTile128x64)
@@ -638,7 +706,7 @@ int run(const Problem& pr) {
     }
   }
   if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
-  if (ar.splitk > 1 && pr.mode == kDense && pl.variant != kVarExact && !is_skinny(pl.variant) && !is_pipelined(pl.variant)) {
+  if (ar.splitk > 1 && pr.mode == kDense && pl.variant != kVarExact && !is_skinny(pl.variant)) {
     const int64_t total = pr.rows * pr.N;
     const int vec_ok = total % 4 == 0 && !misaligned(pr.c, 4 * esz);
     hipLaunchKernelGGL(fp8_splitk_reduce_kernel, dim3(static_cast<unsigned>(ceil_div(ceil_div(total, 4), 256))), dim3(256), 0,

@@ -158,7 +158,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
   int walk_base = 0;
 
   for (int vb = vb_first;; vb += gridDim.x) {
-    int g = 0, mt = 0, nt, m_end, m_first = -1;
+    int g = 0, mt = 0, nt, m_end, m_first = -1, split = 0;
     if (MODE == kMasked) {
       int mtiles = 0;
       while (walk_g < p.G) {
@@ -188,8 +188,13 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       g = p.gidx[m_first];
       m_end = min(p.M, m_first + BM);
     } else {
-      if (vb >= tiles) break;
-      const int t = xcd_remap(vb, tiles);
+      // dense split-K: the K range is cut into p.splitk slices of p.kb_per_split blocks, every (tile, slice) pair is a
+      // unit of work, slices of one tile far apart in the order
+      const int units = MODE == kDense ? tiles * p.splitk : tiles;
+      if (vb >= units) break;
+      const int id = xcd_remap(vb, units);
+      split = MODE == kDense ? id / tiles : 0;
+      const int t = id - split * tiles;
       const int width = p.group_m * tiles_n;
       const int grp = t / width;
       const int first_m = grp * p.group_m;
@@ -208,17 +213,20 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     const int n0 = __builtin_amdgcn_readfirstlane(n_base + nt * BN);
 
     const int64_t esz = p.out_f32 ? 4 : 2;
-    const uint8_t* a_tile = p.a + static_cast<int64_t>(m0) * p.K;
-    const float* as_tile = p.a_s + static_cast<int64_t>(m0) * p.as_sm;
+    const bool sliced = MODE == kDense && p.splitk > 1;
+    const int kb_first = sliced ? split * p.kb_per_split : 0;  // the host leaves no slice empty
+    const uint8_t* a_tile = p.a + static_cast<int64_t>(m0) * p.K + static_cast<int64_t>(kb_first) * kScaleBlock;
+    const float* as_tile = p.a_s + static_cast<int64_t>(m0) * p.as_sm + static_cast<int64_t>(kb_first) * p.as_sk;
     char* c_base = static_cast<char*>(p.c);
     if (MODE == kMasked) {
       a_tile += static_cast<int64_t>(g) * p.a_gs;
       as_tile += static_cast<int64_t>(g) * p.as_gs;
       c_base += static_cast<int64_t>(g) * p.c_gs * esz;
     }
-    const uint8_t* b_tile = p.b + static_cast<int64_t>(g) * p.b_gs + static_cast<int64_t>(n0) * p.K;
+    const uint8_t* b_tile =
+        p.b + static_cast<int64_t>(g) * p.b_gs + static_cast<int64_t>(n0) * p.K + static_cast<int64_t>(kb_first) * kScaleBlock;
     // weight scales: lane i of the wave fetches the scale of the wave's fragment (i & 3) (fragment 0 beyond NF)
-    const float* bs_g = p.b_s + static_cast<int64_t>(g) * p.bs_gs;
+    const float* bs_g = p.b_s + static_cast<int64_t>(g) * p.bs_gs + kb_first;
     const int bs_frag = (lane & 3) < NF ? (lane & 3) : 0;
     const uint32_t bs_off =
         static_cast<uint32_t>(min((n0 + wn0 + 32 * bs_frag) / kScaleBlock, p.nblocks - 1)) * static_cast<uint32_t>(p.kblocks) * 4u;
@@ -326,7 +334,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     constexpr int S = kHoldX ? NF : MF;        // streamed fragments
     constexpr int T = H * S;
     constexpr int kFragBytes = 32 * kScaleBlock;
-    const int nk = p.kblocks;
+    const int nk = sliced ? min(p.kblocks, kb_first + p.kb_per_split) - kb_first : p.kblocks;  // K blocks of this unit
     const int held0 = (kHoldX ? wm0 : Cfg::BM + wn0) * kScaleBlock;      // byte offset of held fragment 0 in a stage
     const int strm0 = (kHoldX ? Cfg::BM + wn0 : wm0) * kScaleBlock;
     constexpr int kScaleOff = Cfg::A_BYTES + Cfg::B_BYTES;
@@ -565,6 +573,27 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     }
 
     // epilogue: lane holds c[m0 + wm0 + 32 mi + (lane & 31)][n0 + wn0 + 32 ni + 8 u + 4 (lane >> 5) + 0..3], u = 0..3
+    if (sliced) {
+      // first pass of split-K: the slice's sums go to the workspace as an fp32 [M][N] matrix of their own;
+      // fp8_splitk_reduce_kernel, launched behind this kernel on the same stream, adds the slices in index order
+      float* mine = p.ws + static_cast<int64_t>(split) * p.M * p.N;
+      const bool vec_ok = (p.N % 4) == 0;
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) {
+        const int m = m0 + wm0 + mi * 32 + l32;
+        if (m >= m_end) continue;
+        float* w_row = mine + static_cast<int64_t>(m) * p.N;
+#pragma unroll
+        for (int ni = 0; ni < NF; ++ni)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int n = n0 + wn0 + ni * 32 + u * 8 + h * 4;
+            const v4f v = {acc[mi][ni][4 * u], acc[mi][ni][4 * u + 1], acc[mi][ni][4 * u + 2], acc[mi][ni][4 * u + 3]};
+            store_row4<true>(w_row, n, v, p.N - n, vec_ok);
+          }
+      }
+      continue;
+    }
     if (p.c_vec16) {
       // bf16 through LDS: stored straight from the accumulator layout every instruction would touch 32 rows with
       // 16 bytes each, partial sectors that the L2 has to merge.  Each wave parks its 64-row tile in its own slice of

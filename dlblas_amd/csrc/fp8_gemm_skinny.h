@@ -23,7 +23,9 @@ struct SkinnyCfg {
   static constexpr int NT = WAVES * 64;
   static constexpr int BN = 16 * NFS;
   static constexpr int RED_BYTES = WAVES * MF * NFS * 64 * 16;
-  static constexpr int DMA_LDS_BYTES = WAVES * UNROLL * (NFS + MF) * 2048 + RED_BYTES;  // staging + reduction
+  static constexpr int STAGING_BYTES = WAVES * UNROLL * (NFS + MF) * 2048;
+  // the reduction buffer reuses the staging areas once every wave is through with its K blocks
+  static constexpr int DMA_LDS_BYTES = STAGING_BYTES > RED_BYTES ? STAGING_BYTES : RED_BYTES;
 };
 
 // 32 operand bytes of one lane for K block `kb`: bytes [16 q, 16 q + 16) and [64 + 16 q, 64 + 16 q + 16) of the
@@ -162,7 +164,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
   constexpr int FRAGS = NFS + MF;                 // 2 KB blocks per K block: weights first, then activations
   constexpr int WAVE_BYTES = U * FRAGS * 2048;    // staging area of one wave
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  v4f(*red)[MF * NFS][64] = reinterpret_cast<v4f(*)[MF * NFS][64]>(smem + WAVES * WAVE_BYTES);
+  v4f(*red)[MF * NFS][64] = reinterpret_cast<v4f(*)[MF * NFS][64]>(smem);  // over the staging areas, behind a barrier
 
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   typedef const __attribute__((address_space(1))) void* global_ptr_t;
@@ -275,6 +277,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
     // the next round of DMA overwrites the staging area: its reads above have returned (their values were used)
   }
 
+  __syncthreads();  // every wave has read its last staged block: the staging areas become the reduction buffer
 #pragma unroll
   for (int mi = 0; mi < MF; ++mi)
 #pragma unroll

@@ -53,7 +53,7 @@ def test_dense_bf16_matches_oracle(dev, M, N, K):
     helpers.tolerance_check(out, ref, f'dense {M}x{N}x{K}')
 
 
-@pytest.mark.parametrize('variant', ['tile128x128', 'tile64x128', 'tile128x64', 'skinny16', 'skinny32', 'skinny64', 'skinny128', 'exact', 'pipe256x128', 'pipe128x256', 'pipe256x256', 'pipe128x256w8', 'pipe256mix'])
+@pytest.mark.parametrize('variant', ['tile128x128', 'tile64x128', 'tile128x64', 'skinny16', 'skinny32', 'skinny64', 'skinny128', 'exact', 'pipe256x128', 'pipe128x256', 'pipe256x256', 'pipe128x256w8', 'pipe256mix', 'pipe128x128', 'pipe128x64'])
 @pytest.mark.parametrize('M,N,K', [(16, 512, 1024), (30, 200, 400), (200, 392, 2048)])
 def test_every_variant(dev, variant, M, N, K):
     print(f'case variant={variant} M={M} N={N} K={K}', flush=True)
@@ -64,7 +64,8 @@ def test_every_variant(dev, variant, M, N, K):
 
 
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize('variant,splitk', [('tile128x128', 2), ('tile128x64', 5), ('tile64x128', 32), (None, 0)])
+@pytest.mark.parametrize('variant,splitk', [('tile128x128', 2), ('tile128x64', 5), ('tile64x128', 32), (None, 0), ('pipe128x256w8', 3),
+                                            ('pipe128x128', 4), ('pipe128x64', 2), ('pipe256x256', 7), ('pipe128x256', 2)])
 @pytest.mark.parametrize('M,N,K', [(128, 2112, 7168), (200, 392, 2048), (129, 130, 1040), (70, 131, 4096)])
 def test_split_k_two_pass(dev, M, N, K, variant, splitk, out_dtype):
     """K split over workgroups: fp32 partial matrices in the workspace, a second kernel adds them in index order.
@@ -84,7 +85,7 @@ def test_split_k_two_pass(dev, M, N, K, variant, splitk, out_dtype):
     assert torch.equal(out, again)
 
 
-@pytest.mark.parametrize('variant', ['pipe256x256', 'pipe128x256w8', 'pipe256mix', 'pipe256x128'])
+@pytest.mark.parametrize('variant', ['pipe256x256', 'pipe128x256w8', 'pipe256mix', 'pipe256x128', 'pipe128x128', 'pipe128x64'])
 @pytest.mark.parametrize('M,N,K', [(200, 392, 2048), (513, 1032, 256)])
 def test_epilogue_through_lds_equals_direct_stores(dev, variant, M, N, K):
     """bf16 results of the pipelined kernels leave through an LDS transpose (whole rows per store instruction) or, by
@@ -100,6 +101,25 @@ def test_epilogue_through_lds_equals_direct_stores(dev, variant, M, N, K):
     staged = _run_dense(dev, a_q, a_s, b_q, b_s, variant=variant)
     assert torch.equal(direct, staged)
     helpers.tolerance_check(staged, orc.dequant_ref(a_q, a_s, b_q, b_s), f'epilogue {variant}')
+
+
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('bn', [0, 4, 12, 20, 28, 32])
+@pytest.mark.parametrize('M,N,K', [(16, 1000, 1024), (5, 130, 256), (40, 2112, 1024), (100, 392, 512)])
+def test_decode_column_split(dev, M, N, K, bn, out_dtype):
+    """Decode kernels with every width of the per-workgroup column range: ranges that are no multiple of 16 straddle
+    weight-scale blocks (128 columns) inside a fragment and end in partly owned fragments; N itself is ragged."""
+    from dlblas_amd import _lib
+    print(f'case decode column split M={M} N={N} K={K} bn={bn} {out_dtype}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=31)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    _lib.tune('skinny_bn', bn)
+    try:
+        out = _run_dense(dev, a_q, a_s, b_q, b_s, dtype=out_dtype)
+    finally:
+        _lib.tune('skinny_bn', 0)
+    assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
+    helpers.tolerance_check(out, ref, f'decode bn={bn} {M}x{N}x{K}')
 
 
 def _random_shapes(n, seed):
