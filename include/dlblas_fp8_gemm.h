@@ -188,8 +188,9 @@ int dlb_fp8_gemm_force_variant(int variant);
 
 /*
  * Tuning / test hook: set knob `knob` for the next calls FROM THIS THREAD; value 0 restores the heuristic.
- *   DLB_KNOB_SPLITK         K slices of the LDS-tiled dense kernels, each summed into its own fp32 matrix in the workspace and added
- *                           by a second kernel in slice order (clamped to what workspace and K allow)
+ *   DLB_KNOB_SPLITK         K slices of the dense tile kernels (all but the decode kernels and the mixed-width launch), each summed
+ *                           into its own fp32 matrix in the workspace and added by a second kernel in slice order (clamped to
+ *                           what workspace and K allow)
  *   DLB_KNOB_SKINNY_WAVES   waves per workgroup of the decode kernels (4, 8 or 16)
  *   DLB_KNOB_SKINNY_UNROLL  K blocks a decode-kernel wave loads before its first MFMA (1, 2 or 4)
  *   DLB_KNOB_SKINNY_NFRAGS  16-row weight fragments per decode workgroup (1 or 2)
