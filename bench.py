@@ -208,6 +208,23 @@ def second_prefill_workload(dev):
              'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes}]
 
 
+def chunked_prefill_workloads(dev):
+    """Dense shapes between decode and prefill (a few hundred rows against the same weight matrices): too few large tiles
+    for the chip, weights streamed from HBM.  Four weight copies in rotation."""
+    import torch
+    rows = []
+    for (M, N, K) in ((256, 7168, 2048), (512, 4096, 7168), (256, 7168, 16384)):
+        a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=4)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        ms = time_call(DenseLauncher(a_q, a_s, ws, out), 100, 10)
+        flops, nbytes = 2.0 * M * N * K, algorithmic_bytes(M, N, K)
+        rows.append({'workload': f'chunk_{M}x{N}x{K}', 'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9,
+                     'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS, 'GBps': nbytes / ms / 1e6,
+                     'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'bytes': nbytes})
+        del a_q, a_s, ws, out
+    return rows
+
+
 def expert_weights(G, N, K, dev, seed):
     import torch
     g = torch.Generator(device=dev).manual_seed(seed)
@@ -461,6 +478,7 @@ def main():
                             'note': '24 distinct weight copies in rotation (353 MB) so reads miss the 256 MB cache'}
         log('grouped workloads')
         others += second_prefill_workload(dev)
+        others += chunked_prefill_workloads(dev)
         others += grouped_workloads(dev)
         others += quantiser_workload(dev)
         others += activation_workloads(dev)

@@ -219,9 +219,10 @@ int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x
   a.topk_is64 = topk_dtype == DLB_IDX_I64, a.start_is64 = start_dtype == DLB_IDX_I64, a.oi_is64 = index_dtype == DLB_IDX_I64;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(a.nblocks)), block(kPermuteThreads);
+  a.fused_scan = static_cast<int64_t>(a.nblocks) * a.E <= kFusedScanMaxInts;
   hipLaunchKernelGGL(ep_scatter_count_kernel, grid, block, static_cast<size_t>(a.E) * sizeof(int), st, a);
   if (int rc = finish("ep_scatter (count)")) return rc;
-  {
+  if (!a.fused_scan) {
     static std::atomic<unsigned long long> lds_done{0};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
@@ -232,9 +233,9 @@ int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x
         return fail(DLB_ERR_LAUNCH, "cannot raise the LDS limit of the scan kernel");
       lds_done.fetch_or(bit, std::memory_order_release);
     }
+    hipLaunchKernelGGL(ep_scatter_scan_kernel, dim3(1), dim3(kScanThreads), kScanTileInts * 4, st, a);
+    if (int rc = finish("ep_scatter (scan)")) return rc;
   }
-  hipLaunchKernelGGL(ep_scatter_scan_kernel, dim3(1), dim3(kScanThreads), kScanTileInts * 4, st, a);
-  if (int rc = finish("ep_scatter (scan)")) return rc;
   hipLaunchKernelGGL(ep_scatter_copy_kernel, grid, dim3(kCopyThreads), 0, st, a);
   return finish("ep_scatter (copy)");
 }

@@ -5,7 +5,8 @@
 // The reference hands out destination rows with one global atomic per (token, slot), in whatever order the atomics
 // resolve.  Here the order is fixed - token-major, slot-minor, the order of the reference's single-program variant
 // (dlblas/kernels/ascend/fused_moe_v3.py:137) - and no global atomic is used: a stable counting sort in three
-// launches (per-block histograms, scan, rank + copy).  The copies are HBM-bound: every source row is read once and
+// launches (per-block histograms, scan, rank + copy; the scan launch is dropped while the histogram matrix is small
+// enough for every copy block to sum the rows of the blocks before it itself).  The copies are HBM-bound: every source row is read once and
 // written once per valid slot, 16 bytes per lane.
 #pragma once
 
@@ -43,6 +44,7 @@ struct ScatterArgs {
   int64_t T, m_len;
   int H, E, topk_n, tokens_per_block, nblocks;
   int topk_is64, start_is64, oi_is64;
+  int fused_scan;  // the copy kernel derives the block's first rows from the raw histograms itself (no scan launch)
 };
 
 // Expert id of entry `i` (token-major) of block `b`, or -1.
@@ -144,9 +146,14 @@ __global__ void __launch_bounds__(kScanThreads) ep_scatter_scan_kernel(const Sca
 // tokens to their destination rows.  Every block also fills its slice of m_indices.
 constexpr int kCopyThreads = 1024;
 
+constexpr int kFusedScanMaxInts = 32768;  // histogram entries up to which a copy block scans for itself
+
 __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const ScatterArgs p) {
   __shared__ int ids[kPermuteThreads];
   __shared__ int64_t dest[kPermuteThreads];
+  __shared__ int64_t excl_l[kScanMaxExperts + 1];  // fused scan: exclusive prefix sum of counts
+  __shared__ int64_t base_l[kScanMaxExperts];      //             first row this block writes for every expert
+  __shared__ int psum[kCopyThreads];
   const int tid = threadIdx.x;
   const int b = blockIdx.x;
   int id = -1;
@@ -154,13 +161,52 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
     id = scatter_entry_id(p, b, tid);
     ids[tid] = id;
   }
+  if (p.fused_scan) {
+    // what the scan launch would have left in start_excl and block_hist[b][.], computed by every block for itself:
+    // the first wave scans counts 64 at a time, then all threads add up the histogram rows of the blocks before b
+    if (tid < 64) {
+      int64_t carry = 0;
+      for (int e0 = 0; e0 < p.E; e0 += 64) {
+        const int e = e0 + tid;
+        const int64_t c = e < p.E ? max(p.counts[e], 0) : 0;
+        int64_t incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+          const int64_t up = __shfl_up(incl, off);
+          if (tid >= off) incl += up;
+        }
+        if (e < p.E) excl_l[e] = carry + incl - c;
+        carry += __shfl(incl, 63);
+      }
+      if (tid == 0) excl_l[p.E] = carry;
+    }
+    const int cols = min(p.E, kCopyThreads);
+    const int P = kCopyThreads / cols;
+    const int my_part = tid / cols, my_col = tid % cols;
+    for (int c0 = 0; c0 < p.E; c0 += cols) {
+      const int e = c0 + my_col;
+      int s_rows = 0;
+      if (my_part < P && e < p.E)
+        for (int r = my_part; r < b; r += P) s_rows += p.block_hist[static_cast<int64_t>(r) * p.E + e];
+      psum[tid] = s_rows;
+      __syncthreads();  // also orders excl_l
+      if (my_part == 0 && e < p.E) {
+        int64_t first = excl_l[e];
+        for (int q = 0; q < P; ++q) first += psum[q * cols + my_col];
+        base_l[e] = first;
+        if (b == static_cast<int>(gridDim.x) - 1)  // the last block knows every expert's first free row after the call
+          store_index(p.start_loc, p.start_is64, e, first + p.block_hist[static_cast<int64_t>(b) * p.E + e]);
+      }
+      __syncthreads();
+    }
+  }
   __syncthreads();
   if (tid < kPermuteThreads) {
     int64_t d = -1;
     if (id >= 0) {
       int rank = 0;
       for (int j = 0; j < tid; ++j) rank += (ids[j] == id);
-      d = static_cast<int64_t>(p.block_hist[static_cast<int64_t>(b) * p.E + id]) + rank;
+      d = (p.fused_scan ? base_l[id] : static_cast<int64_t>(p.block_hist[static_cast<int64_t>(b) * p.E + id])) + rank;
       const int64_t t = static_cast<int64_t>(b) * p.tokens_per_block + tid / p.topk_n;
       store_index(p.out_index, p.oi_is64, t * p.oi_s0 + (tid % p.topk_n) * p.oi_s1, d);
     }
@@ -170,14 +216,15 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
 
   // m_indices: rows [0, start_excl[E]) in slices over the blocks; expert of a row by binary search
   {
-    const int64_t total = min(p.start_excl[p.E], p.m_len);
+    const int64_t* excl = p.fused_scan ? excl_l : p.start_excl;
+    const int64_t total = min(excl[p.E], p.m_len);
     const int64_t per = (total + gridDim.x - 1) / gridDim.x;
     const int64_t r1 = min(total, (b + 1) * per);
     for (int64_t r = b * per + tid; r < r1; r += kCopyThreads) {
       int lo = 0, hi = p.E;  // largest e with start_excl[e] <= r
       while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (p.start_excl[mid] <= r)
+        if (excl[mid] <= r)
           lo = mid;
         else
           hi = mid;

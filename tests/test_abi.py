@@ -42,6 +42,16 @@ def test_error_codes_match_header():
         assert getattr(_lib, f'ERR_{name}') == value
 
 
+def test_knob_ids_match_header():
+    header = open(HEADER).read()
+    ids = {m.group(1).lower(): int(m.group(2)) for m in re.finditer(r'#define DLB_KNOB_([A-Z_]+) (\d+)', header)}
+    assert ids == _lib.KNOBS
+    lib = _lib.load()
+    for knob in ids.values():
+        assert lib.dlb_fp8_gemm_tune(knob, 0) == 0
+    assert lib.dlb_fp8_gemm_tune(max(ids.values()) + 1, 0) == _lib.ERR_BAD_SHAPE and 'knob' in _lib.last_error()
+
+
 def test_host_only_entry_points():
     lib = _lib.load()
     assert _lib.variant_names()[0] == 'exact' and 'tile128x128' in _lib.variant_names()

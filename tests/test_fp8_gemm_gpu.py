@@ -37,6 +37,7 @@ DENSE_SHAPES = [
     (1, 7168, 2048), (16, 7168, 2048), (64, 7168, 2048), (128, 7168, 2048),
     (1, 2112, 7168), (16, 2112, 7168), (64, 2112, 7168), (128, 2112, 7168),
     (300, 2112, 1536),    # ragged M and N tiles
+    (256, 7168, 2048), (384, 2112, 7168), (130, 7168, 16384),  # between decode and prefill: small tiles, K split over workgroups
     (129, 130, 384),      # N not a multiple of 4: scalar stores
     (33, 200, 400),       # K tail (400 = 3 * 128 + 16)
     (17, 64, 200),        # K not a multiple of 16: exact path

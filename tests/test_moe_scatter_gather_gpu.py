@@ -73,7 +73,9 @@ def test_scatter_reference_test_construction(dev):
 
 
 @pytest.mark.parametrize('index_dtype,start_dtype,strided', [(torch.int64, torch.int32, False), (torch.int32, torch.int64, True)])
-@pytest.mark.parametrize('T,H,E,topk', [(1, 128, 1, 1), (300, 1024, 8, 8), (1000, 7168, 32, 8), (257, 256, 40, 3), (50, 512, 300, 64)])
+@pytest.mark.parametrize('T,H,E,topk', [(1, 128, 1, 1), (300, 1024, 8, 8), (1000, 7168, 32, 8), (257, 256, 40, 3), (50, 512, 300, 64),
+                                       (100, 128, 1100, 8),    # more experts than threads in the in-kernel scan
+                                       (700, 128, 1500, 8)])   # histogram matrix too large for it: separate scan launch
 def test_scatter_matches_oracle(dev, T, H, E, topk, index_dtype, start_dtype, strided):
     print(f'case scatter T={T} H={H} E={E} topk={topk} {index_dtype} {start_dtype} strided={strided}', flush=True)
     g = helpers.gen(T + H + E)
