@@ -654,6 +654,7 @@ int run(const Problem& pr) {
         // the real tile count is only known on the device; cover the worst case with a resident-sized grid
         const int64_t worst = static_cast<int64_t>(ar.tiles_m) * ar.tiles_n * pr.G;
         grid = worst < static_cast<int64_t>(cus) * 4 ? worst : static_cast<int64_t>(cus) * 4;
+        grid = (grid + 31) / 32 * 32;  // the ring kernels deal tiles to the XCDs four at a time
       }
       if (grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)grid);
       const int g = static_cast<int>(grid);

@@ -160,18 +160,25 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
   for (int vb = vb_first;; vb += gridDim.x) {
     int g = 0, mt = 0, nt, m_end, m_first = -1, split = 0;
     if (MODE == kMasked) {
+      // The tile count is only known on the device, so the grid is persistent; the hardware deals consecutive
+      // workgroups to the 8 XCDs in turn.  Of every 32 consecutive tiles each XCD takes 4 consecutive ones: the row
+      // tiles of an expert, which are adjacent in the order and read the same weight tile, meet in one L2, and the
+      // last, partial round still spreads over all XCDs (the grid is a multiple of 32).
+      const int grid = static_cast<int>(gridDim.x);
+      const int w = vb % grid;
+      const int tile_id = vb - w + (w / 32) * 32 + (w % 8) * 4 + (w / 8) % 4;
       int mtiles = 0;
       while (walk_g < p.G) {
         const int valid = min(max(p.gidx[walk_g], 0), p.M);
         mtiles = (valid + BM - 1) / BM;
         const int cnt = mtiles * tiles_n;
-        if (vb < walk_base + cnt) break;
+        if (tile_id < walk_base + cnt) break;
         walk_base += cnt;
         ++walk_g;
       }
       if (walk_g >= p.G) break;
       g = walk_g;
-      const int local = vb - walk_base;
+      const int local = tile_id - walk_base;
       mt = local % mtiles;
       nt = local / mtiles;
       m_end = min(max(p.gidx[g], 0), p.M);
