@@ -123,6 +123,28 @@ def test_decode_column_split(dev, M, N, K, bn, out_dtype):
     helpers.tolerance_check(out, ref, f'decode bn={bn} {M}x{N}x{K}')
 
 
+@pytest.mark.parametrize('ws_bytes', [0, 65536 + 4096])
+@pytest.mark.parametrize('M,N,K', [(128, 2112, 7168), (300, 2112, 1536), (16, 512, 1024)])
+def test_c_abi_without_a_usable_workspace(dev, M, N, K, ws_bytes):
+    """Straight through the C ABI with no workspace or one too small for anything: no re-laid scales, no K split,
+    the same results."""
+    import ctypes
+    from dlblas_amd import _lib
+    print(f'case no workspace M={M} N={N} K={K} ws_bytes={ws_bytes}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=17)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    a, b, sa, sb = a_q.to(dev), b_q.to(dev), a_s.to(dev), b_s.to(dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    vp = ctypes.c_void_p
+    rc = _lib.load().dlb_fp8_gemm(vp(a.data_ptr()), vp(b.data_ptr()), vp(sa.data_ptr()), vp(sb.data_ptr()), vp(out.data_ptr()),
+                                  M, N, K, sa.stride(0), sa.stride(1), _lib.OUT_BF16, vp(ws.data_ptr() if ws_bytes else 0), ws_bytes,
+                                  vp(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    helpers.tolerance_check(out, ref, f'no workspace {M}x{N}x{K}')
+
+
 def _random_shapes(n, seed):
     import random
     rng = random.Random(seed)
