@@ -37,6 +37,7 @@ SYMBOLS = {
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
     'dlb_fp8_gemm_tune': (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
+    'dlb_fp8_gemm_plan': (ctypes.c_int, [ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_sz, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 3),
     'dlb_silu_mul': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp] + [_c_i64] * 4 + [_c_vp]),
     'dlb_silu_mul_quant': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
     'dlb_silu_mul_quant_masked': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp, _c_vp] + [_c_i64] * 6 + [_c_vp]),
@@ -121,6 +122,15 @@ def variant_names():
             return names
         names.append(name.decode())
         i += 1
+
+
+def plan(mode: int, rows: int, N: int, K: int, workspace_bytes: int = None, compute_units: int = 256):
+    """(variant name, K slices, decode columns per workgroup) the library would use; touches no GPU."""
+    lib = load()
+    v, s, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    ws = WORKSPACE_BYTES if workspace_bytes is None else workspace_bytes
+    check(lib.dlb_fp8_gemm_plan(mode, rows, N, K, ws, compute_units, ctypes.byref(v), ctypes.byref(s), ctypes.byref(c)))
+    return variant_names()[v.value], s.value, c.value
 
 
 def force_variant(name_or_id) -> None:

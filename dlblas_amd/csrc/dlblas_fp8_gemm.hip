@@ -834,6 +834,19 @@ int dlb_fp8_quant_128x128(const void* w, int w_dtype, void* q, float* s, int64_t
   return DLB_OK;
 }
 
+int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t workspace_bytes, int compute_units, int* variant,
+                      int* k_slices, int* decode_columns) {
+  dlb::clear_error();
+  if (mode < dlb::kDense || mode > dlb::kMasked) return dlb::fail(DLB_ERR_BAD_SHAPE, "mode %d is not 0 (dense), 1 (contiguous) or 2 (masked)", mode);
+  if (rows < 0 || N < 0 || K < 0) return dlb::fail(DLB_ERR_BAD_SHAPE, "negative dimension (rows=%lld, N=%lld, K=%lld)", (long long)rows, (long long)N, (long long)K);
+  if (compute_units <= 0) return dlb::fail(DLB_ERR_BAD_SHAPE, "compute_units must be positive");
+  const dlb::Plan pl = dlb::make_plan(mode, rows, N, K, compute_units, workspace_bytes);
+  if (variant) *variant = pl.variant;
+  if (k_slices) *k_slices = pl.splitk;
+  if (decode_columns) *decode_columns = dlb::is_skinny(pl.variant) ? pl.sk_bn : 0;
+  return DLB_OK;
+}
+
 int dlb_fp8_gemm_force_variant(int variant) {
   if (variant >= dlb::kVarCount) return dlb::fail(DLB_ERR_BAD_SHAPE, "unknown kernel variant %d", variant);
   dlb::g_forced_variant = variant < 0 ? -1 : variant;

@@ -180,6 +180,17 @@ int dlb_fp8_quant_128x128(const void* w, int w_dtype, void* q, float* s, int64_t
                           int64_t w_row_stride, float eps, void* stream);
 
 /*
+ * Host-only query: what the library would launch for a problem, without launching anything (no GPU is touched).
+ * mode 0 = dlb_fp8_gemm, 1 = grouped contiguous (rows = M_sum), 2 = grouped masked (rows = M_max); `compute_units`
+ * is the CU count to plan for (256 on MI355X).  Outputs (each may be NULL): the kernel variant id
+ * (dlb_fp8_gemm_variant_name), the number of K slices summed in a second pass (1 = none), the output columns per
+ * workgroup of the decode kernels (0 for other variants).  Honours the calling thread's forced variant and knobs, as
+ * a launch would.  No counterpart in the reference, whose single Triton configuration needs no plan.
+ */
+int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t workspace_bytes, int compute_units, int* variant,
+                      int* k_slices, int* decode_columns);
+
+/*
  * Tuning / test hook: force the kernel variant the next calls FROM THIS THREAD use.
  * variant < 0 restores the built-in shape heuristic.  Returns DLB_ERR_BAD_SHAPE for an unknown id.
  * Variant ids are listed by dlb_fp8_gemm_variant_name().
