@@ -145,6 +145,26 @@ def test_c_abi_without_a_usable_workspace(dev, M, N, K, ws_bytes):
     helpers.tolerance_check(out, ref, f'no workspace {M}x{N}x{K}')
 
 
+@pytest.mark.parametrize('M,N,K', [(0, 512, 1024), (16, 0, 1024), (16, 512, 0), (300, 392, 0)])
+def test_empty_dimensions(dev, M, N, K):
+    """No rows or no columns: an empty result; no K: a sum over nothing, i.e. zeros."""
+    from dlblas_amd.kernels.fp8_gemm import fp8_gemm
+    print(f'case empty M={M} N={N} K={K}', flush=True)
+    a = torch.zeros(M, K, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    b = torch.zeros(N, K, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    a_s = torch.ones(M, (K + 127) // 128, device=dev)
+    b_s = torch.ones((N + 127) // 128, (K + 127) // 128, device=dev)
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        out = fp8_gemm(a, b, a_s, b_s)
+    finally:
+        torch.set_default_dtype(prev)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (M, N) and out.dtype == torch.bfloat16
+    assert (out == 0).all()
+
+
 def _random_shapes(n, seed):
     import random
     rng = random.Random(seed)
