@@ -658,10 +658,13 @@ int run(const Problem& pr) {
       }
       if (grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)grid);
       const int g = static_cast<int>(grid);
+      // Dense launches of many rounds of equal tiles run one resident workgroup per CU that walks its tiles itself
+      // (the ring kernels loop over tiles anyway): saves the hardware's per-workgroup start, 4 % at six rounds.
+      const int g_dense = pr.mode == kDense && grid >= 4ll * cus ? cus : g;
       if (pl.variant == kVarPipe256mix) {
         const int64_t split = pick_mixed_split(pr.rows, pr.N, cus);
         if (split >= pr.N) {
-          e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g, dev, pr.stream);
+          e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
         } else {
           static std::atomic<unsigned long long> lds_done{0};
           auto kernel = fp8_gemm_pipelined_mixed_kernel<Pipe256x256, Pipe256x192>;
@@ -681,7 +684,7 @@ int run(const Problem& pr) {
       else if (pl.variant == kVarPipe128x256)
         e = launch_pipelined_mode<Pipe128x256>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe256x256)
-        e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g, dev, pr.stream);
+        e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
       else if (pl.variant == kVarPipe128x256w8 && tile_list) {
         static std::atomic<unsigned long long> lds_done{0};
         auto kernel = fp8_gemm_contig_list_kernel<Pipe256x256, Pipe128x256w8>;
@@ -693,7 +696,7 @@ int run(const Problem& pr) {
           e = hipGetLastError();
         }
       } else if (pl.variant == kVarPipe128x256w8)
-        e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g, dev, pr.stream);
+        e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g_dense, dev, pr.stream);
       else if (pl.variant == kVarPipe128x128)
         e = launch_pipelined_mode<Pipe128x128>(pr.mode, ar, g, dev, pr.stream);
       else if (pl.variant == kVarPipe128x64)
