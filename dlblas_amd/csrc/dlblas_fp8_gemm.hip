@@ -270,13 +270,14 @@ int64_t pick_mixed_split(int64_t M, int64_t N, int cus) {
   const int64_t tm = ceil_div(M, 256);
   const double narrow_cost = 0.78;  // 192 / 256 of the work plus the fixed per-tile part
   int64_t best_split = N;
-  double best = mixed_makespan(tm * ceil_div(N, 256), 0, narrow_cost, cus);
+  const double uniform = mixed_makespan(tm * ceil_div(N, 256), 0, narrow_cost, cus);
+  double best = uniform;
   if (tm * ceil_div(N, 256) <= 16 * static_cast<int64_t>(cus)) {  // many rounds: the tail no longer matters
     for (int64_t ca = N / 256; ca >= 0; --ca) {
       const int64_t split = ca * 256;
       if (split >= N) continue;
       const double t = mixed_makespan(tm * ca, tm * ceil_div(N - split, 192), narrow_cost, cus);
-      if (t < best - 1e-6) best = t, best_split = split;
+      if (t < best - 1e-6 && t < 0.96 * uniform) best = t, best_split = split;  // a uniform launch of many rounds runs resident, worth 4 %
     }
   }
   memo[memo_next] = Memo{M, N, cus, best_split};
