@@ -403,6 +403,17 @@ def measured_traffic(workload):
         return None
 
 
+def copy_calibration(dev):
+    """Three 1 GiB device copies: the kernel of known size that the HBM counters of a profiled run are scaled by."""
+    import torch
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -414,6 +425,9 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run three 1 GiB device copies: the known-size kernel that HBM counters are scaled by')
     ap.add_argument('--no-other', action='store_true', help='skip the decode sweep and the grouped workloads')
+    ap.add_argument('--grouped-only', action='store_true',
+                    help='run only the two grouped MoE workloads and print their rows (the command the rocprofv3 summaries of '
+                    'the grouped kernels are made with)')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1', file=sys.stderr)
@@ -428,6 +442,13 @@ def main():
     torch.cuda.set_device(dev)
     if args.variant:
         _lib.force_variant(args.variant)
+
+    if args.grouped_only:
+        rows = grouped_workloads(dev)
+        if args.copy_calibration:
+            copy_calibration(dev)
+        print(json.dumps({'grouped_workloads': rows}), flush=True)
+        return
 
     kind, M, N, K = WORKLOADS[args.workload]
     log(f'workload {args.workload}: generating inputs')
@@ -486,12 +507,7 @@ def main():
         result['other_workloads'] = others
 
     if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        copy_calibration(dev)
 
     if not args.no_cpu_baseline:
         log('cpu baseline')
