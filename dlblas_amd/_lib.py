@@ -16,6 +16,7 @@ ABI_VERSION = 1
 OUT_BF16, OUT_F32 = 0, 1
 WS_COUNTER_BYTES = 65536
 WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
+STATIC_SCRATCH_BYTES = 16 << 20  # DLB_STATIC_SCRATCH_BYTES: the array dlb_fp8_gemm_noalloc works in
 
 ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_BAD_STRIDE, ERR_BAD_DTYPE, ERR_WORKSPACE, ERR_ALIGNMENT, ERR_LAUNCH = \
     -1, -2, -3, -4, -5, -6, -7
@@ -28,6 +29,7 @@ SYMBOLS = {
     'dlb_last_error': (ctypes.c_char_p, []),
     'dlb_fp8_gemm_workspace_bytes': (_c_sz, [_c_i64, _c_i64, _c_i64]),
     'dlb_fp8_gemm': (ctypes.c_int, [_c_vp] * 5 + [_c_i64] * 5 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
+    'dlb_fp8_gemm_noalloc': (ctypes.c_int, [_c_vp] * 5 + [_c_i64] * 5 + [ctypes.c_int, _c_vp]),
     'dlb_fp8_gemm_grouped_contiguous':
     (ctypes.c_int, [_c_vp] * 6 + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 2 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_grouped_masked':

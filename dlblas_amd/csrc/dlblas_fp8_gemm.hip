@@ -18,6 +18,13 @@
 #include "fp8_gemm_tiled.h"
 #include "fp8_quant.h"
 
+// Scratch for dlb_fp8_gemm_noalloc: device memory that is part of the loaded code object, so a caller that cannot
+// allocate (HIP graph capture, a serving loop that forbids hipMalloc) needs no workspace of its own.  Every GPU the
+// library runs on holds its own copy at its own address until the process ends.  The name is only a host-side
+// handle: host code uses the per-device address hipGetSymbolAddress returns (static_scratch_ptr below), never the
+// name itself.
+static __device__ __align__(256) unsigned char scratch[DLB_STATIC_SCRATCH_BYTES];
+
 namespace dlb {
 
 // ---------------------------------------------------------------------------------------------------------
@@ -492,8 +499,10 @@ struct Problem {
 };
 
 
-int run(const Problem& pr) {
+// Argument checks that need no device.  Returns DLB_OK with *empty set when there is nothing to compute.
+int check_problem(const Problem& pr, bool* empty) {
   g_err[0] = '\0';
+  *empty = false;
   if (pr.out_dtype != DLB_OUT_BF16 && pr.out_dtype != DLB_OUT_F32)
     return fail(DLB_ERR_BAD_DTYPE, "out_dtype %d is neither DLB_OUT_BF16 nor DLB_OUT_F32", pr.out_dtype);
   if (pr.rows < 0 || pr.N < 0 || pr.K < 0)
@@ -505,7 +514,10 @@ int run(const Problem& pr) {
                 (long long)pr.N, (long long)pr.K);
   if (pr.mode != kDense && pr.G < 0) return fail(DLB_ERR_BAD_SHAPE, "negative group count %d", pr.G);
   const int64_t groups = pr.mode == kDense ? 1 : pr.G;
-  if (pr.rows == 0 || pr.N == 0 || groups == 0) return DLB_OK;
+  if (pr.rows == 0 || pr.N == 0 || groups == 0) {
+    *empty = true;
+    return DLB_OK;
+  }
   if (!pr.c) return fail(DLB_ERR_NULL_POINTER, "c is NULL");
   if (pr.mode != kDense && !pr.gidx)
     return fail(DLB_ERR_NULL_POINTER, "%s is NULL", pr.mode == kContiguous ? "m_indices" : "masked_m");
@@ -526,6 +538,15 @@ int run(const Problem& pr) {
     return fail(DLB_ERR_ALIGNMENT, "a and b must be 16-byte aligned");
   if (misaligned(pr.c, 2) || misaligned(pr.a_s, 4) || misaligned(pr.b_s, 4))
     return fail(DLB_ERR_ALIGNMENT, "c / a_s / b_s are not aligned to their element size");
+  return DLB_OK;
+}
+
+int run(const Problem& pr) {
+  bool empty = false;
+  const int bad = check_problem(pr, &empty);
+  if (bad != DLB_OK || empty) return bad;
+  const int64_t groups = pr.mode == kDense ? 1 : pr.G;
+  const int64_t kblocks = ceil_div(pr.K, kScaleBlock);
 
   int dev = 0;
   const int cus = device_cu_count(&dev);
@@ -722,6 +743,23 @@ int run(const Problem& pr) {
   return DLB_OK;
 }
 
+// Device address of `scratch` on the current device, looked up once per device (with that device current) and kept.
+int static_scratch_ptr(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<void*> ptr_of[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
+  if (dev < 0 || dev >= kMaxDevices) return fail(DLB_ERR_LAUNCH, "device ordinal %d beyond the %d this library tracks", dev, kMaxDevices);
+  void* ptr = ptr_of[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return fail(DLB_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+    ptr_of[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return DLB_OK;
+}
+
 }  // namespace
 }  // namespace dlb
 
@@ -751,6 +789,29 @@ int dlb_fp8_gemm(const void* a, const void* b, const float* a_s, const float* b_
                  size_t workspace_bytes, void* stream) {
   dlb::Problem pr{dlb::kDense, a, b, a_s, b_s, c, nullptr, M, N, K, 1, 0, as_stride_m, as_stride_k, out_dtype,
                   workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  return dlb::run(pr);
+}
+
+int dlb_fp8_gemm_noalloc(const void* a, const void* b, const float* a_s, const float* b_s, void* c, int64_t M, int64_t N,
+                         int64_t K, int64_t as_stride_m, int64_t as_stride_k, int out_dtype, void* stream) {
+  dlb::Problem pr{dlb::kDense, a, b, a_s, b_s, c, nullptr, M, N, K, 1, 0, as_stride_m, as_stride_k, out_dtype,
+                  nullptr, 0, static_cast<hipStream_t>(stream)};
+  bool empty = false;
+  const int bad = dlb::check_problem(pr, &empty);
+  if (bad != DLB_OK || empty) return bad;
+  // the one hard requirement on the scratch: the activation scales, re-laid rows-contiguous, have to fit behind the
+  // reserved head (the K slices of the split-K plans adapt to whatever is left)
+  const int64_t relaid = dlb::ceil_div(K, dlb::kScaleBlock) * ((M + 3) / 4 * 4) * static_cast<int64_t>(sizeof(float));
+  if (relaid > static_cast<int64_t>(DLB_STATIC_SCRATCH_BYTES) - DLB_WS_COUNTER_BYTES - 256)
+    return dlb::fail(DLB_ERR_WORKSPACE,
+                     "M=%lld x ceil(K/128)=%lld needs %lld bytes of re-laid scales, the static scratch holds %lld; use dlb_fp8_gemm "
+                     "with a workspace", (long long)M, (long long)dlb::ceil_div(K, dlb::kScaleBlock), (long long)relaid,
+                     (long long)(static_cast<int64_t>(DLB_STATIC_SCRATCH_BYTES) - DLB_WS_COUNTER_BYTES - 256));
+  void* ws = nullptr;
+  const int rc = dlb::static_scratch_ptr(&ws);
+  if (rc != DLB_OK) return rc;
+  pr.ws = ws;
+  pr.ws_bytes = DLB_STATIC_SCRATCH_BYTES;
   return dlb::run(pr);
 }
 

@@ -95,6 +95,28 @@ int dlb_fp8_gemm(const void* a, const void* b, const float* a_s, const float* b_
                  int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * dlb_fp8_gemm for callers that cannot allocate device memory and have no workspace to pass: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its Triton launch
+ * needs no scratch).  Same operands, same kernels and same results as dlb_fp8_gemm called with a workspace of
+ * DLB_STATIC_SCRATCH_BYTES bytes; the scratch (re-laid activation scales, fp32 partial sums of the split-K plans) is
+ * a fixed array inside the library's code object, DLB_STATIC_SCRATCH_BYTES per GPU, held by every GPU the library
+ * runs on until the process ends.  The call allocates and frees nothing and does not synchronise.
+ *
+ *   - Limit: 4 * ceil(K/128) * M bytes (M rounded up to a multiple of 4) must fit in DLB_STATIC_SCRATCH_BYTES minus
+ *     the reserved head (64 KiB + 256); larger problems are rejected with DLB_ERR_WORKSPACE and nothing is enqueued.
+ *   - All calls on one GPU share that GPU's array and overwrite what the previous call left in it (nothing in it has
+ *     to be zero at entry): calls that may overlap in time on one GPU - different streams - race; order them or use
+ *     dlb_fp8_gemm with a workspace per stream.
+ *   - The first call on a device looks up the array's device address (hipGetSymbolAddress); make that call outside
+ *     a graph capture.
+ */
+#define DLB_STATIC_SCRATCH_BYTES (16u << 20)
+int dlb_fp8_gemm_noalloc(const void* a, const void* b, const float* a_s, const float* b_s, void* c,
+                         int64_t M, int64_t N, int64_t K,
+                         int64_t as_stride_m, int64_t as_stride_k,
+                         int out_dtype, void* stream);
+
+/*
  * Grouped GEMM, expert-contiguous rows.  Replaces deep_gemm.m_grouped_fp8_gemm_nt_contiguous
  * (call site dlblas/kernels/fused_moe_v3.py:235-245, buffers built at :262-308).
  *
