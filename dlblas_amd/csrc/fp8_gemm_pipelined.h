@@ -15,10 +15,6 @@
 #include "fp8_gemm_common.h"
 #include "fp8_gemm_tiled.h"  // xcd_remap
 
-#ifndef DLB_EXP
-#define DLB_EXP 0  // tuning builds set bits to cut pieces out of the K loop and time what is left (results are wrong)
-#endif
-
 namespace dlb {
 
 // D = A_op * B_op^T, A_op / B_op [32 x 64] e4m3: lane l supplies row (l & 31), 32 K-bytes selected by (l >> 5).
@@ -497,26 +493,22 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         const int si = t / H, hi = t % H;
         if (si == S - 1 && hi == 0) {
           // every LDS read of this stage has been issued and the barrier waits for their return: hand it over
-          if (!(DLB_EXP & 8)) {
-            wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
-            lds_barrier();
-          }
+          wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
+          lds_barrier();
         }
-        if (!(DLB_EXP & 1)) {
-          if (t >= kP) {
-            if (t - kP < kSlots) {
-              if (t - kP == 0) issue_slot(std::integral_constant<int, 0>{}, kb_new, stage);
-              if (t - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_new, stage);
-              if (t - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_new, stage);
-              if (t - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_new, stage);
-              if (t - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_new, stage);
-            }
-          } else if (t + T - kP < kSlots) {
-            if (t + T - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_prev, prev_stage);
-            if (t + T - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_prev, prev_stage);
-            if (t + T - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_prev, prev_stage);
-            if (t + T - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_prev, prev_stage);
+        if (t >= kP) {
+          if (t - kP < kSlots) {
+            if (t - kP == 0) issue_slot(std::integral_constant<int, 0>{}, kb_new, stage);
+            if (t - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_new, stage);
+            if (t - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_new, stage);
+            if (t - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_new, stage);
+            if (t - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_new, stage);
           }
+        } else if (t + T - kP < kSlots) {
+          if (t + T - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_prev, prev_stage);
+          if (t + T - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_prev, prev_stage);
+          if (t + T - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_prev, prev_stage);
+          if (t + T - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_prev, prev_stage);
         }
         // The scheduling fences pin the order MFMA pair -> reloads -> scale FMAs; without them the compiler
         // hoists the reloads above the MFMAs into fresh registers and the kernel spills.
@@ -534,11 +526,11 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         }
         __builtin_amdgcn_sched_barrier(0);
         // in-place reloads: the MFMAs above were the last readers of these registers
-        if (hi == H - 1 && si + 1 < S && !(DLB_EXP & 4)) {
+        if (hi == H - 1 && si + 1 < S) {
           sf[0] = lds_read_frag32(smem, cur_base + strm0 + (si + 1) * kFragBytes, lc, 0);
           sf[1] = lds_read_frag32(smem, cur_base + strm0 + (si + 1) * kFragBytes, lc, 1);
         }
-        if (si == S - 1 && !(DLB_EXP & 4)) {
+        if (si == S - 1) {
           hf[hi][0] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 0);
           hf[hi][1] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 1);
           if (hi == 0) load_scales(nxt_base, sc_next);
@@ -548,10 +540,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
           }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (DLB_EXP & 2) {
-          const int mi = kHoldX ? hi : si, ni = kHoldX ? si : hi;
-          acc[mi][ni][0] += part[t & kSlot][t & 15];
-        } else if (Cfg::PARTS == 1) {
+        if (Cfg::PARTS == 1) {
           // scale-and-accumulate this tile; the other wave of the SIMD owns the matrix pipe meanwhile
           const int mi = kHoldX ? hi : si, ni = kHoldX ? si : hi;
           acc[mi][ni] += part[0] * sc[mi][kUniformW ? 0 : ni];

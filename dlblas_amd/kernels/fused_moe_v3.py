@@ -43,8 +43,7 @@ def ep_scatter(
     """recv_x [T, H] fp8 and recv_x_scale [T, H / 128] are copied to output_tensor / output_tensor_scale so that the
     rows of each expert are adjacent; m_indices [rows] gets the expert of every reserved row, output_index [T, topk]
     the destination row of every routed slot, expert_start_loc [E] the first free row of every expert."""
-    BLOCK_E = 128  # token num of per expert is aligned to 128
-    assert m_indices.shape[0] % BLOCK_E == 0
+    assert m_indices.shape[0] % 128 == 0, 'every expert span is a whole number of 128-row GEMM blocks'
     assert recv_x.dim() == 2 and recv_topk.dim() == 2 and recv_x.shape[0] == recv_topk.shape[0]
     assert recv_x.stride(1) == 1 and output_tensor.stride(1) == 1, 'rows must be contiguous'
     if recv_x.dtype != torch.float8_e4m3fn or output_tensor.dtype != torch.float8_e4m3fn:
@@ -86,32 +85,39 @@ def fused_moe_v3(
     w2_weight_fp8: Tuple[torch.Tensor, torch.Tensor],
     num_recv_tokens_per_expert: Optional[List[int]],
 ):
-    """scatter -> grouped GEMM (gate/up) -> silu * up + quantise -> grouped GEMM (down) -> weighted gather."""
-    hidden_states_fp8, hidden_states_scale = hidden_states_fp8
-    if num_recv_tokens_per_expert is None:
-        return hidden_states_fp8.to(torch.bfloat16)
-    all_tokens = sum(num_recv_tokens_per_expert)
-    if all_tokens <= 0:
-        return hidden_states_fp8.to(torch.bfloat16)
-    M, K = hidden_states_fp8.size()
-    N = w13_weight_fp8[0].size(1)
-    dev = hidden_states_fp8.device
-    gather_out = torch.empty((M, K), device=dev, dtype=torch.bfloat16)
-    # padding rows are computed by the GEMMs like any other row; zero them so that no NaN pattern left in the
-    # allocation reaches the quantiser between the two GEMMs
-    input_tensor = torch.zeros((all_tokens, K), device=dev, dtype=torch.uint8).view(hidden_states_fp8.dtype)
-    input_tensor_scale = torch.zeros((all_tokens, K // 128), device=dev, dtype=torch.float32)
-    m_indices = torch.empty(all_tokens, device=dev, dtype=torch.int32)
-    output_index = torch.empty_like(topk_idx)
-    num_recv_tokens_per_expert_gpu = torch.tensor(num_recv_tokens_per_expert, dtype=torch.int32, pin_memory=True,
-                                                  device='cpu').to(dev, non_blocking=True)
-    expert_start_loc = torch.empty_like(num_recv_tokens_per_expert_gpu)
-    ep_scatter(hidden_states_fp8, hidden_states_scale, topk_idx, num_recv_tokens_per_expert_gpu, expert_start_loc,
-               input_tensor, input_tensor_scale, m_indices, output_index)
-    gateup_output = torch.empty((all_tokens, N), device=dev, dtype=torch.bfloat16)
-    m_grouped_fp8_gemm_nt_contiguous((input_tensor, input_tensor_scale), w13_weight_fp8, gateup_output, m_indices)
-    down_input_fp8, down_input_scale = silu_and_mul_post_quant(gateup_output, 128)
-    down_output = torch.empty((all_tokens, K), device=dev, dtype=torch.bfloat16)
-    m_grouped_fp8_gemm_nt_contiguous((down_input_fp8, down_input_scale), w2_weight_fp8, down_output, m_indices)
-    ep_gather(down_output, topk_idx, topk_weights, output_index, gather_out)
-    return gather_out
+    """One expert-parallel MLP over the tokens this GPU received: rows are sorted by expert (ep_scatter), pass through
+    gate/up GEMM -> silu(gate) * up with 1 x 128 re-quantisation -> down GEMM as expert-contiguous grouped GEMMs, and
+    come back to token order as the routing-weighted sum of each token's slots (ep_gather).  Signature and early
+    returns of the reference driver (dlblas/kernels/fused_moe_v3.py:246-343); every intermediate is allocated here,
+    per call, as there."""
+    tokens_q, tokens_scale = hidden_states_fp8
+    rows_total = 0 if num_recv_tokens_per_expert is None else sum(num_recv_tokens_per_expert)
+    if rows_total <= 0:
+        return tokens_q.to(torch.bfloat16)  # nothing routed to a local expert: the caller gets its input back in bf16
+    n_tokens, hidden = tokens_q.shape
+    inter2 = w13_weight_fp8[0].size(1)  # gate and up halves side by side
+    dev = tokens_q.device
+
+    def buf(shape, dtype, zero=False):
+        return (torch.zeros if zero else torch.empty)(shape, device=dev, dtype=dtype)
+
+    # Expert-sorted activations.  The spans are padded to 128 rows per expert and the GEMMs compute the padding like
+    # any other row, so it starts as zeros: stale bytes of the allocator must not reach the quantiser as NaN.
+    sorted_q = buf((rows_total, hidden), torch.uint8, zero=True).view(tokens_q.dtype)
+    sorted_scale = buf((rows_total, hidden // 128), torch.float32, zero=True)
+    row_expert = buf((rows_total, ), torch.int32)
+    slot_row = torch.empty_like(topk_idx)
+    per_expert = torch.tensor(num_recv_tokens_per_expert, dtype=torch.int32, pin_memory=True).to(dev, non_blocking=True)
+    first_row = torch.empty_like(per_expert)
+    ep_scatter(tokens_q, tokens_scale, topk_idx, per_expert, first_row, sorted_q, sorted_scale, row_expert, slot_row)
+
+    gate_up = buf((rows_total, inter2), torch.bfloat16)
+    m_grouped_fp8_gemm_nt_contiguous((sorted_q, sorted_scale), w13_weight_fp8, gate_up, row_expert)
+    act_q, act_scale = silu_and_mul_post_quant(gate_up, 128)
+    del gate_up
+    down = buf((rows_total, hidden), torch.bfloat16)
+    m_grouped_fp8_gemm_nt_contiguous((act_q, act_scale), w2_weight_fp8, down, row_expert)
+
+    combined = buf((n_tokens, hidden), torch.bfloat16)
+    ep_gather(down, topk_idx, topk_weights, slot_row, combined)
+    return combined

@@ -20,3 +20,19 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if 'gpu' in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Relative error at the strict floor (|ref| floored at 1e-3 rms) of every parity check that ran: reported, not
+    asserted (the asserted bars are in helpers.tolerance_check)."""
+    try:
+        import helpers
+    except ImportError:
+        return
+    log = helpers.strict_floor_log
+    if not log:
+        return
+    worst = sorted(log, key=lambda kv: -kv[1])[:12]
+    terminalreporter.write_line(f'parity checks against the exact oracle: {len(log)}; largest relative errors at the 1e-3 rms floor:')
+    for what, err in worst:
+        terminalreporter.write_line(f'  {err:.3e}  {what}')

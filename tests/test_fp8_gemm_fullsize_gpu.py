@@ -3,7 +3,6 @@
 import pytest
 import torch
 
-import bench
 import helpers
 from oracle import fp8_block_gemm as orc
 
@@ -35,8 +34,7 @@ def _sample_rows(M, count, seed):
 @pytest.mark.parametrize('M,N,K', [(4096, 7168, 18432), (4096, 24576, 1536)])
 def test_prefill_full_size(dev, M, N, K):
     print(f'case prefill full size M={M} N={N} K={K}', flush=True)
-    a_q, a_s, weights = bench.make_inputs(M, N, K, dev)
-    b_q, b_s = weights[0]
+    a_q, a_s, b_q, b_s = helpers.make_dense_device(M, N, K, dev)
     out = _gemm(a_q, b_q, a_s, b_s)
     torch.cuda.synchronize()
     rows = _sample_rows(M, 48, 1)
@@ -55,24 +53,12 @@ def test_prefill_full_size(dev, M, N, K):
 @pytest.mark.parametrize('N,K', [(7168, 2048), (2112, 7168)])
 def test_decode_full_size(dev, M, N, K):
     print(f'case decode full size M={M} N={N} K={K}', flush=True)
-    a_q, a_s, weights = bench.make_inputs(M, N, K, dev)
-    b_q, b_s = weights[0]
+    a_q, a_s, b_q, b_s = helpers.make_dense_device(M, N, K, dev)
     out = _gemm(a_q, b_q, a_s, b_s)
     torch.cuda.synchronize()
     ref = orc.dequant_ref(a_q.cpu(), a_s.cpu(), b_q.cpu(), b_s.cpu())
     helpers.tolerance_check(out, ref, f'decode {M}x{N}x{K}')
     assert torch.equal(_gemm(a_q, b_q, a_s * 0.5, b_s), out * 0.5)
-
-
-def _expert_weights(G, N, K, dev, seed):
-    g = torch.Generator(device=dev).manual_seed(seed)
-    qs, ss = [], []
-    for _ in range(G):
-        w = (torch.randn(N, K, device=dev, generator=g) * 0.02).to(torch.bfloat16)
-        q, s = bench.quantise_weight(w)
-        qs.append(q)
-        ss.append(s)
-    return torch.stack(qs), torch.stack(ss)
 
 
 def test_grouped_contiguous_full_size(dev):
@@ -91,8 +77,8 @@ def test_grouped_contiguous_full_size(dev):
     gd = torch.Generator(device=dev).manual_seed(21)
     a = torch.randn(M_sum, K, device=dev, generator=gd).to(torch.bfloat16)
     a[~valid.to(dev)] = 0
-    a_q, a_s = bench.quantise_act(a)
-    w_q, w_s = _expert_weights(G, N, K, dev, 22)
+    a_q, a_s = helpers.quantise_act_device(a)
+    w_q, w_s = helpers.expert_weights_device(G, N, K, dev, 22)
     out = torch.full((M_sum, N), 3.0, dtype=torch.bfloat16, device=dev)
     m_grouped_fp8_gemm_nt_contiguous((a_q, a_s), (w_q, w_s), out, m_indices.to(dev))
     torch.cuda.synchronize()
@@ -120,7 +106,7 @@ def test_grouped_masked_full_size(dev):
     masked_m = torch.randint(0, M_max + 1, (G, ), generator=g, dtype=torch.int32)
     gd = torch.Generator(device=dev).manual_seed(23)
     a = torch.randn(G * M_max, K, device=dev, generator=gd).to(torch.bfloat16)
-    a_q, a_s = bench.quantise_act(a)
+    a_q, a_s = helpers.quantise_act_device(a)
     a_q, a_s = a_q.reshape(G, M_max, K), a_s.reshape(G, M_max, K // 128).clone()
     bits = a_q.view(torch.uint8).clone()
     garbage = torch.randint(0, 256, bits.shape, device=dev, generator=gd, dtype=torch.uint8)  # includes NaN codes
@@ -128,7 +114,7 @@ def test_grouped_masked_full_size(dev):
     bits[beyond] = garbage[beyond]
     a_s[beyond] = float('nan')
     a_q = bits.view(torch.float8_e4m3fn)
-    w_q, w_s = _expert_weights(G, N, K, dev, 24)
+    w_q, w_s = helpers.expert_weights_device(G, N, K, dev, 24)
     sentinel = -7.0
     out = torch.full((G, M_max, N), sentinel, dtype=torch.bfloat16, device=dev)
     m_grouped_fp8_gemm_nt_masked((a_q, a_s), (w_q, w_s), out, masked_m.to(dev), int(masked_m.float().mean()))
