@@ -12,7 +12,7 @@ import torch
 
 from ._build import LIB_PATH
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 OUT_BF16, OUT_F32 = 0, 1
 WS_COUNTER_BYTES = 65536
 WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
@@ -39,7 +39,8 @@ SYMBOLS = {
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
     'dlb_fp8_gemm_tune': (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
-    'dlb_fp8_gemm_plan': (ctypes.c_int, [ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_sz, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 3),
+    'dlb_fp8_gemm_plan': (ctypes.c_int, [ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_sz, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 3 +
+                          [ctypes.POINTER(_c_i64)]),
     'dlb_silu_mul': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp] + [_c_i64] * 4 + [_c_vp]),
     'dlb_silu_mul_quant': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
     'dlb_silu_mul_quant_masked': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp, _c_vp] + [_c_i64] * 6 + [_c_vp]),
@@ -115,6 +116,26 @@ def workspace(device: torch.device, stream_handle: int) -> torch.Tensor:
     return buf
 
 
+def prepare(device=None, stream=None) -> None:
+    """Do now, on (device, stream), everything a first call would do lazily: load the library, allocate the workspace
+    of that (device, stream) pair and look up the device address of the static scratch of dlb_fp8_gemm_noalloc (one tiny
+    GEMM through it).  Call it before capturing a HIP graph on `stream` or entering a loop that must not allocate; the
+    calls captured or made afterwards allocate nothing in this package (torch still allocates outputs that the callee
+    owns).  `stream` is a torch.cuda.Stream (default: the current one)."""
+    lib = load()
+    dev = torch.device('cuda', torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(dev):
+        st = torch.cuda.current_stream(dev) if stream is None else stream
+        with torch.cuda.stream(st):
+            workspace(dev, st.cuda_stream)
+            a = torch.zeros(16, 128, dtype=torch.uint8, device=dev)
+            s = torch.ones(16, 1, dtype=torch.float32, device=dev)
+            c = torch.empty(16, 16, dtype=torch.float32, device=dev)
+            check(lib.dlb_fp8_gemm_noalloc(_ptr(a), _ptr(a), _ptr(s), _ptr(s), _ptr(c), 16, 16, 128, 1, 1, OUT_F32,
+                                           ctypes.c_void_p(st.cuda_stream)))
+        st.synchronize()
+
+
 def variant_names():
     lib = load()
     names, i = [], 0
@@ -128,11 +149,17 @@ def variant_names():
 
 def plan(mode: int, rows: int, N: int, K: int, workspace_bytes: int = None, compute_units: int = 256):
     """(variant name, K slices, decode columns per workgroup) the library would use; touches no GPU."""
+    return plan_full(mode, rows, N, K, workspace_bytes, compute_units)[:3]
+
+
+def plan_full(mode: int, rows: int, N: int, K: int, workspace_bytes: int = None, compute_units: int = 256):
+    """plan() plus the first column of the narrow tiles of the mixed-width prefill launch (N: all tiles equal)."""
     lib = load()
-    v, s, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    v, s, c, n = ctypes.c_int(), ctypes.c_int(), ctypes.c_int(), ctypes.c_int64()
     ws = WORKSPACE_BYTES if workspace_bytes is None else workspace_bytes
-    check(lib.dlb_fp8_gemm_plan(mode, rows, N, K, ws, compute_units, ctypes.byref(v), ctypes.byref(s), ctypes.byref(c)))
-    return variant_names()[v.value], s.value, c.value
+    check(lib.dlb_fp8_gemm_plan(mode, rows, N, K, ws, compute_units, ctypes.byref(v), ctypes.byref(s), ctypes.byref(c),
+                                ctypes.byref(n)))
+    return variant_names()[v.value], s.value, c.value, n.value
 
 
 def force_variant(name_or_id) -> None:

@@ -4,9 +4,6 @@
 #include "../../include/dlblas_fp8_moe.h"
 
 #include <atomic>
-#include <functional>
-#include <queue>
-#include <vector>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -34,23 +31,24 @@ namespace dlb {
 // ---------------------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) fp8_gemm_exact_kernel(const Args p) {
   const int n = blockIdx.x * 64 + (threadIdx.x & 63);
-  const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
-  if (m >= p.M || n >= p.N) return;
-  const uint8_t* a_row = p.a + static_cast<int64_t>(m) * p.K;
+  if (n >= p.N) return;
   const uint8_t* b_row = p.b + static_cast<int64_t>(n) * p.K;
-  const float* as_row = p.a_s + static_cast<int64_t>(m) * p.as_sm;
   const float* bs_row = p.b_s + static_cast<int64_t>(n / kScaleBlock) * p.kblocks;
-  float acc = 0.f;
-  for (int kb = 0; kb < p.kblocks; ++kb) {
-    const int k1 = min(p.K, (kb + 1) * kScaleBlock);
-    float dot = 0.f;
-    for (int k = kb * kScaleBlock; k < k1; ++k) dot = fmaf(e4m3_to_f32(a_row[k]), e4m3_to_f32(b_row[k]), dot);
-    acc += dot * as_row[static_cast<int64_t>(kb) * p.as_sk] * bs_row[kb];
+  for (int64_t m = blockIdx.y * 4 + (threadIdx.x >> 6); m < p.M; m += static_cast<int64_t>(gridDim.y) * 4) {
+    const uint8_t* a_row = p.a + m * p.K;
+    const float* as_row = p.a_s + m * p.as_sm;
+    float acc = 0.f;
+    for (int kb = 0; kb < p.kblocks; ++kb) {
+      const int k1 = min(p.K, (kb + 1) * kScaleBlock);
+      float dot = 0.f;
+      for (int k = kb * kScaleBlock; k < k1; ++k) dot = fmaf(e4m3_to_f32(a_row[k]), e4m3_to_f32(b_row[k]), dot);
+      acc += dot * as_row[static_cast<int64_t>(kb) * p.as_sk] * bs_row[kb];
+    }
+    if (p.out_f32)
+      static_cast<float*>(p.c)[m * p.N + n] = acc;
+    else
+      static_cast<__bf16*>(p.c)[m * p.N + n] = static_cast<__bf16>(acc);
   }
-  if (p.out_f32)
-    static_cast<float*>(p.c)[static_cast<int64_t>(m) * p.N + n] = acc;
-  else
-    static_cast<__bf16*>(p.c)[static_cast<int64_t>(m) * p.N + n] = static_cast<__bf16>(acc);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -108,8 +106,6 @@ enum Variant : int {
   kVarSkinny32,
   kVarSkinny64,
   kVarSkinny128,
-  kVarPipe256x128,
-  kVarPipe128x256,
   kVarPipe256x256,
   kVarPipe128x256w8,
   kVarPipe256mix,
@@ -119,14 +115,12 @@ enum Variant : int {
 };
 
 const char* const kVariantNames[kVarCount] = {
-    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "skinny64", "skinny128", "pipe256x128", "pipe128x256", "pipe256x256", "pipe128x256w8", "pipe256mix", "pipe128x128", "pipe128x64",
+    "exact", "tile128x128", "tile64x128", "tile128x64", "skinny16", "skinny32", "skinny64", "skinny128", "pipe256x256", "pipe128x256w8", "pipe256mix", "pipe128x128", "pipe128x64",
 };
 
 typedef TileCfg<128, 128, 2, 2> Tile128x128;
 typedef TileCfg<64, 128, 2, 2> Tile64x128;
 typedef TileCfg<128, 64, 2, 2> Tile128x64;
-typedef PipeCfg<2, 2, 4, 2, 3, 2, true> Pipe256x128;  // 4 waves, wave tile 128 x 64, register double buffering
-typedef PipeCfg<2, 2, 2, 4, 3, 2, true> Pipe128x256;  // 4 waves, wave tile 64 x 128
 typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256;  // 8 waves, wave tile 64 x 128
 typedef PipeCfg<4, 2, 2, 3, 2, 2> Pipe256x192;  // narrow tiles of the mixed-width launch
 typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
@@ -191,11 +185,11 @@ hipError_t launch_pipelined_mode(int mode, const Args& args, int grid, int dev, 
 }
 
 template <class Cfg>
-hipError_t launch_skinny_cfg(const Args& args, int dev, hipStream_t stream) {
+hipError_t launch_skinny_cfg(bool dma, const Args& args, int dev, hipStream_t stream) {
   static std::atomic<unsigned long long> lds_done{0}, lds_done_tail{0}, lds_done_dma{0};
   const bool ktail = args.K % kScaleBlock != 0;
   // full-line DMA staging where it fits in LDS and K has no ragged block; else the register-load kernel
-  if (!ktail && Cfg::DMA_LDS_BYTES <= 160 * 1024 && g_knob[kKnobSkinnyDma] != 2) {
+  if (dma && !ktail && Cfg::DMA_LDS_BYTES <= 160 * 1024 && g_knob[kKnobSkinnyDma] != 2) {
     auto kernel = fp8_gemm_skinny_dma_kernel<Cfg>;
     hipError_t e = ensure_lds(kernel, Cfg::DMA_LDS_BYTES, dev, &lds_done_dma);
     if (e != hipSuccess) return e;
@@ -212,83 +206,83 @@ hipError_t launch_skinny_cfg(const Args& args, int dev, hipStream_t stream) {
 
 // Skinny kernel instances: MF in {1, 2}, (waves, unroll) in a small set, n fragments in {1, 2}.
 template <int MF, int NFS>
-hipError_t launch_skinny_wu(int waves, int unroll, const Args& args, int dev, hipStream_t stream) {
+hipError_t launch_skinny_wu(int waves, int unroll, bool dma, const Args& args, int dev, hipStream_t stream) {
   if (waves >= 16) {
-    if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 16, 4, NFS>>(args, dev, stream);
-    if (unroll >= 2) return launch_skinny_cfg<SkinnyCfg<MF, 16, 2, NFS>>(args, dev, stream);
-    return launch_skinny_cfg<SkinnyCfg<MF, 16, 1, NFS>>(args, dev, stream);
+    if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 16, 4, NFS>>(dma, args, dev, stream);
+    if (unroll >= 2) return launch_skinny_cfg<SkinnyCfg<MF, 16, 2, NFS>>(dma, args, dev, stream);
+    return launch_skinny_cfg<SkinnyCfg<MF, 16, 1, NFS>>(dma, args, dev, stream);
   }
   if (waves >= 8) {
-    if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 8, 4, NFS>>(args, dev, stream);
-    if (unroll >= 2) return launch_skinny_cfg<SkinnyCfg<MF, 8, 2, NFS>>(args, dev, stream);
-    return launch_skinny_cfg<SkinnyCfg<MF, 8, 1, NFS>>(args, dev, stream);
+    if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 8, 4, NFS>>(dma, args, dev, stream);
+    if (unroll >= 2) return launch_skinny_cfg<SkinnyCfg<MF, 8, 2, NFS>>(dma, args, dev, stream);
+    return launch_skinny_cfg<SkinnyCfg<MF, 8, 1, NFS>>(dma, args, dev, stream);
   }
-  if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 4, 4, NFS>>(args, dev, stream);
-  return launch_skinny_cfg<SkinnyCfg<MF, 4, 2, NFS>>(args, dev, stream);
+  if (unroll >= 4) return launch_skinny_cfg<SkinnyCfg<MF, 4, 4, NFS>>(dma, args, dev, stream);
+  return launch_skinny_cfg<SkinnyCfg<MF, 4, 2, NFS>>(dma, args, dev, stream);
 }
 
 // Large activation blocks (M up to 64 / 128) keep to one K block in flight per wave: their fragments fill the registers.
 template <int MF, int NFS>
-hipError_t launch_skinny_big(int waves, const Args& args, int dev, hipStream_t stream) {
-  if (waves >= 16) return launch_skinny_cfg<SkinnyCfg<MF, 16, 1, NFS>>(args, dev, stream);
-  if (waves >= 8) return launch_skinny_cfg<SkinnyCfg<MF, 8, 1, NFS>>(args, dev, stream);
-  return launch_skinny_cfg<SkinnyCfg<MF, 4, 1, NFS>>(args, dev, stream);
+hipError_t launch_skinny_big(int waves, bool dma, const Args& args, int dev, hipStream_t stream) {
+  if (waves >= 16) return launch_skinny_cfg<SkinnyCfg<MF, 16, 1, NFS>>(dma, args, dev, stream);
+  if (waves >= 8) return launch_skinny_cfg<SkinnyCfg<MF, 8, 1, NFS>>(dma, args, dev, stream);
+  return launch_skinny_cfg<SkinnyCfg<MF, 4, 1, NFS>>(dma, args, dev, stream);
 }
 
-hipError_t launch_skinny(int mf, int nfs, int waves, int unroll, const Args& args, int dev, hipStream_t stream) {
+hipError_t launch_skinny(int mf, int nfs, int waves, int unroll, bool dma, const Args& args, int dev, hipStream_t stream) {
   switch (mf) {
     case 1:
-      return nfs == 2 ? launch_skinny_wu<1, 2>(waves, unroll, args, dev, stream)
-                      : launch_skinny_wu<1, 1>(waves, unroll, args, dev, stream);
+      return nfs == 2 ? launch_skinny_wu<1, 2>(waves, unroll, dma, args, dev, stream)
+                      : launch_skinny_wu<1, 1>(waves, unroll, dma, args, dev, stream);
     case 2:
-      return nfs == 2 ? launch_skinny_wu<2, 2>(waves, unroll, args, dev, stream)
-                      : launch_skinny_wu<2, 1>(waves, unroll, args, dev, stream);
+      return nfs == 2 ? launch_skinny_wu<2, 2>(waves, unroll, dma, args, dev, stream)
+                      : launch_skinny_wu<2, 1>(waves, unroll, dma, args, dev, stream);
     case 4:
-      return nfs == 2 ? launch_skinny_big<4, 2>(waves, args, dev, stream) : launch_skinny_big<4, 1>(waves, args, dev, stream);
+      return nfs == 2 ? launch_skinny_big<4, 2>(waves, dma, args, dev, stream) : launch_skinny_big<4, 1>(waves, dma, args, dev, stream);
     default:
-      return nfs == 2 ? launch_skinny_big<8, 2>(waves, args, dev, stream) : launch_skinny_big<8, 1>(waves, args, dev, stream);
+      return nfs == 2 ? launch_skinny_big<8, 2>(waves, dma, args, dev, stream) : launch_skinny_big<8, 1>(waves, dma, args, dev, stream);
   }
 }
 
 
-// Makespan (in units of one 256 x 256 tile) of `ta` tiles of cost 1 followed by `tb` tiles of cost `cb`, handed
-// out in order, each to the worker that becomes free first.
+// Makespan (in units of one 256 x 256 tile) of `ta` tiles of cost 1 followed by `tb` tiles of cost `cb` < 1, handed
+// out in order, each to the worker that becomes free first.  After the unit tiles `ra = ta % workers` workers are busy
+// until qa + 1 and the others until qa = ta / workers; every later tile starts at one of the times qa + j cb (on one
+// of the workers - ra early ones) or qa + 1 + j cb (on one of the ra late ones), smallest first, so the last start is
+// found by merging two arithmetic sequences: a few steps per round of workgroups instead of one heap operation per tile.
 double mixed_makespan(int64_t ta, int64_t tb, double cb, int workers) {
-  std::priority_queue<double, std::vector<double>, std::greater<double>> free_at;
-  for (int i = 0; i < workers; ++i) free_at.push(0.0);
-  double end = 0.0;
-  for (int64_t t = 0; t < ta + tb; ++t) {
-    const double done = free_at.top() + (t < ta ? 1.0 : cb);
-    free_at.pop();
-    free_at.push(done);
-    if (done > end) end = done;
+  const int64_t qa = ta / workers, ra = ta % workers;
+  const int64_t n_early = workers - ra, n_late = ra;
+  double end = ta > 0 ? static_cast<double>(qa + (ra > 0 ? 1 : 0)) : 0.0;
+  int64_t left = tb, i = 0, j = 0;
+  while (left > 0) {
+    const double t_early = static_cast<double>(qa) + static_cast<double>(i) * cb;
+    const double t_late = static_cast<double>(qa + 1) + static_cast<double>(j) * cb;
+    const bool take_early = n_late == 0 || t_early <= t_late;
+    const int64_t n = take_early ? n_early : n_late;
+    const double start = take_early ? t_early : t_late;
+    (take_early ? i : j) += 1;
+    left -= n < left ? n : left;
+    if (start + cb > end) end = start + cb;
   }
   return end;
 }
 
 // Columns [0, n_split) in 256-wide tiles, the rest in 192-wide tiles; returns n_split (== N: no narrow region).
+// Cost: (N / 256 + 1) candidate cuts x a few steps per round, a few microseconds at most, no state.
 int64_t pick_mixed_split(int64_t M, int64_t N, int cus) {
-  // the search simulates a few thousand tile hand-outs: remember the answers of the shapes seen by this thread
-  struct Memo { int64_t M, N; int cus; int64_t split; };
-  thread_local Memo memo[8] = {};
-  thread_local int memo_next = 0;
-  for (const Memo& m : memo)
-    if (m.M == M && m.N == N && m.cus == cus && m.M > 0) return m.split;
   const int64_t tm = ceil_div(M, 256);
   const double narrow_cost = 0.78;  // 192 / 256 of the work plus the fixed per-tile part
   int64_t best_split = N;
+  if (tm * ceil_div(N, 256) > 16 * static_cast<int64_t>(cus)) return N;  // many rounds: the tail no longer matters
   const double uniform = mixed_makespan(tm * ceil_div(N, 256), 0, narrow_cost, cus);
   double best = uniform;
-  if (tm * ceil_div(N, 256) <= 16 * static_cast<int64_t>(cus)) {  // many rounds: the tail no longer matters
-    for (int64_t ca = N / 256; ca >= 0; --ca) {
-      const int64_t split = ca * 256;
-      if (split >= N) continue;
-      const double t = mixed_makespan(tm * ca, tm * ceil_div(N - split, 192), narrow_cost, cus);
-      if (t < best - 1e-6 && t < 0.96 * uniform) best = t, best_split = split;  // a uniform launch of many rounds runs resident, worth 4 %
-    }
+  for (int64_t ca = N / 256; ca >= 0; --ca) {
+    const int64_t split = ca * 256;
+    if (split >= N) continue;
+    const double t = mixed_makespan(tm * ca, tm * ceil_div(N - split, 192), narrow_cost, cus);
+    if (t < best - 1e-6 && t < 0.96 * uniform) best = t, best_split = split;  // a uniform launch of many rounds runs resident, worth 4 %
   }
-  memo[memo_next] = Memo{M, N, cus, best_split};
-  memo_next = (memo_next + 1) % 8;
   return best_split;
 }
 
@@ -298,6 +292,7 @@ struct Plan {
   int splitk;
   int sk_waves, sk_unroll, sk_nfrags;  // skinny kernel shape
   int sk_bn;                           // columns per workgroup of its DMA-staged form
+  bool sk_dma;                         // decode kernels may use the DMA-staged form
 };
 
 void tile_dims(int variant, int* bm, int* bn) {
@@ -320,10 +315,6 @@ void tile_dims(int variant, int* bm, int* bn) {
     case kVarSkinny128:
       *bm = 128, *bn = 16;
       break;
-    case kVarPipe256x128:
-      *bm = 256, *bn = 128;
-      break;
-    case kVarPipe128x256:
     case kVarPipe128x256w8:
       *bm = 128, *bn = 256;
       break;
@@ -341,7 +332,7 @@ void tile_dims(int variant, int* bm, int* bn) {
 
 bool is_skinny(int v) { return v >= kVarSkinny16 && v <= kVarSkinny128; }
 int skinny_rows(int v) { return 16 << (v - kVarSkinny16); }
-bool is_pipelined(int v) { return v >= kVarPipe256x128 && v <= kVarPipe128x64; }
+bool is_pipelined(int v) { return v >= kVarPipe256x256 && v <= kVarPipe128x64; }
 
 // Split count no larger than `want` whose slices hold at least two K blocks and whose fp32 partial matrices fit.
 int clamp_splitk(int want, int64_t M, int64_t N, int kblocks, size_t avail) {
@@ -399,8 +390,10 @@ MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_av
   return best;
 }
 
-Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes) {
-  Plan pl{kVarTile128x128, 128, 128, 1, 4, 4, 1, 16};
+// dma_ok: the DMA kernels address their sources with 32-bit byte offsets from the tile's first row (up to 256 rows x K
+// bytes, 512 scale rows x stride); false sends such problems to the kernels with 64-bit addressing.
+Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes, bool dma_ok) {
+  Plan pl{kVarTile128x128, 128, 128, 1, 4, 4, 1, 16, dma_ok};
   const int kblocks = static_cast<int>(ceil_div(K, kScaleBlock));
   const size_t ws_avail = ws_bytes > DLB_WS_COUNTER_BYTES ? ws_bytes - DLB_WS_COUNTER_BYTES : 0;
   int mid_splitk = 0;  // K slices chosen together with a DMA-ring variant
@@ -440,8 +433,7 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
     }
   }
   if (K % 16 != 0) v = kVarExact;
-  if (is_pipelined(v) && (K % kScaleBlock != 0 || K == 0)) v = kVarTile128x128;  // DMA path moves whole K blocks
-  if (v == kVarPipe256x128 && mode == kContiguous) v = kVarPipe128x256;       // a tile must not straddle experts
+  if (is_pipelined(v) && (K % kScaleBlock != 0 || K == 0 || !dma_ok)) v = kVarTile128x128;  // DMA path moves whole K blocks
   if ((v == kVarPipe256x256 || v == kVarPipe256mix) && mode == kContiguous) v = kVarPipe128x256w8;
   if (v == kVarPipe256mix && mode != kDense) v = kVarPipe256x256;
   if (is_skinny(v) && (mode != kDense || M > skinny_rows(v))) v = kVarTile128x128;
@@ -449,6 +441,10 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
   pl.variant = v;
   tile_dims(v, &pl.bm, &pl.bn);
   if (mode == kDense && is_pipelined(v) && mid_splitk > 1) pl.splitk = mid_splitk;
+  // tuning knob: a K slice count for the dense tile kernels (twice the block count lets clamp_splitk go down to one
+  // block per slice)
+  const bool knob_splitk = g_knob[kKnobSplitK] > 0 && mode == kDense && v != kVarExact && !is_skinny(v) && v != kVarPipe256mix;
+  if (knob_splitk) pl.splitk = clamp_splitk(g_knob[kKnobSplitK], M, N, kblocks * 2, ws_avail);
   if (mode != kDense || v == kVarExact || is_pipelined(v) || (kblocks < 2 && !is_skinny(v))) return pl;
 
   const int64_t tiles_n = ceil_div(N, pl.bn);
@@ -457,7 +453,7 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
     // K is split over the waves of a workgroup only.  Pick the wave count so that every wave has two or so K
     // blocks and the unroll so that a wave issues all of its loads before its first MFMA.
     int waves = kblocks >= 8 ? 8 : 4;
-    if (g_knob[kKnobSkinnyWaves] > 0) waves = g_knob[kKnobSkinnyWaves];
+    if (g_knob[kKnobSkinnyWaves] > 0) waves = g_knob[kKnobSkinnyWaves] >= 16 ? 16 : (g_knob[kKnobSkinnyWaves] >= 8 ? 8 : 4);
     const int per_wave = static_cast<int>(ceil_div(kblocks, waves));
     // measured on MI355X: one K block in flight per wave is as good as more once eight waves share a row block
     int unroll = waves >= 8 ? 1 : (per_wave >= 3 ? 4 : 2);
@@ -473,13 +469,85 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
       pl.sk_nfrags = pl.sk_bn > 16 ? 2 : 1;
     }
     pl.bn = 16 * pl.sk_nfrags;
-  } else {
+    // the reduction buffer (waves x fragments x 1 KB) has to fit the 160 KB of LDS whatever the knobs ask for
+    const int frags = skinny_rows(v) / 16 * pl.sk_nfrags;
+    while (pl.sk_waves > 4 && pl.sk_waves * frags * 1024 > 160 * 1024) pl.sk_waves /= 2;
+  } else if (!knob_splitk) {
     // few tiles and a long K: split K over workgroups (partial sums in the workspace, second pass adds them)
     const int64_t tiles = ceil_div(M, pl.bm) * tiles_n;
     if (tiles * 2 > cus) return pl;
     pl.splitk = clamp_splitk(static_cast<int>(cus / tiles), M, N, kblocks, avail);  // one workgroup per CU: a single round
   }
   return pl;
+}
+
+// Everything the host decides about one launch, from shapes, strides and the workspace size alone: run() launches
+// exactly this and dlb_fp8_gemm_plan reports it.
+struct Resolved {
+  Plan pl;
+  int splitk, kb_per_split;  // K slices summed in a second pass (1 = none), K blocks per slice
+  bool tile_list;            // expert-contiguous rows: device-built list of 256- and 128-row tiles
+  int64_t nblk;              //   128-row blocks it covers
+  bool relayout;             // activation scales re-laid rows-contiguous in the workspace first
+  int64_t rows_pad;          //   rows per K block of the re-laid copy
+  size_t ws_used;            // bytes of the workspace's data region taken by list and scales; partial sums follow
+  int64_t n_split;           // mixed-width launch: first column of the 192-wide tiles (N: uniform 256-wide tiles)
+  int64_t grid;              // workgroups of the main kernel
+  bool resident;             // dense launch of many rounds: one resident workgroup per CU walks the tiles
+};
+
+Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as_sm, int64_t as_sk, bool have_ws,
+                 size_t ws_bytes, int cus) {
+  Resolved r{};
+  const int64_t kblocks = ceil_div(K, kScaleBlock);
+  const int64_t groups = mode == kDense ? 1 : G;
+  const bool dma_ok = K < (1ll << 24) && as_sm < (1ll << 21);
+  const bool usable_ws = have_ws && ws_bytes > DLB_WS_COUNTER_BYTES;
+  r.pl = make_plan(mode, rows, N, K, cus, usable_ws ? ws_bytes : 0, dma_ok);
+  const Plan& pl = r.pl;
+  const int want = usable_ws ? pl.splitk : 1;
+  r.kb_per_split = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, want));
+  r.splitk = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, r.kb_per_split));  // no empty slice
+  r.n_split = N;
+  if (mode == kContiguous && pl.variant == kVarPipe128x256w8 && g_forced_variant < 0 && usable_ws && kblocks > 0) {
+    const int64_t nblk = ceil_div(rows, kScaleBlock);
+    const size_t bytes = (static_cast<size_t>(2 + 2 * nblk) * sizeof(int32_t) + 255) / 256 * 256;
+    if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
+  }
+  if (is_pipelined(pl.variant) && as_sk == 1 && as_sm > 1 && usable_ws && kblocks > 1) {
+    // row-major activation scales: re-lay them rows-contiguous in the workspace first (a few microseconds) so the
+    // GEMM fetches 8 cache lines of scales per K step and tile instead of 256
+    const int64_t rows_pad = (rows + 3) / 4 * 4;
+    const int64_t need = groups * kblocks * rows_pad * static_cast<int64_t>(sizeof(float));
+    if (static_cast<size_t>(need) + r.ws_used + DLB_WS_COUNTER_BYTES <= ws_bytes && rows_pad * kblocks < (1ll << 31)) {
+      r.relayout = true, r.rows_pad = rows_pad;
+      r.ws_used += (static_cast<size_t>(need) + 255) / 256 * 256;
+    }
+  }
+  if (r.splitk > 1 && is_pipelined(pl.variant)) {
+    // the partial matrices of the K slices follow whatever else lives in the workspace; fewer slices if they do not fit
+    const size_t avail = ws_bytes - DLB_WS_COUNTER_BYTES - r.ws_used;
+    const size_t per_slice = static_cast<size_t>(rows) * N * sizeof(float);
+    if (per_slice * r.splitk > avail) {
+      const int fit = per_slice > 0 && avail / per_slice >= 1 ? static_cast<int>(avail / per_slice) : 1;
+      r.kb_per_split = static_cast<int>(ceil_div(kblocks, fit));
+      r.splitk = static_cast<int>(ceil_div(kblocks, r.kb_per_split));
+    }
+  }
+  if (pl.variant == kVarPipe256mix) r.n_split = pick_mixed_split(rows, N, cus);
+  const int64_t tiles_m = ceil_div(rows, pl.bm), tiles_n = ceil_div(N, pl.bn);
+  int64_t grid = tiles_m * tiles_n * r.splitk;
+  if (mode == kMasked) {
+    // the real tile count is only known on the device; cover the worst case with a resident-sized grid
+    const int64_t worst = tiles_m * tiles_n * G;
+    grid = worst < static_cast<int64_t>(cus) * 4 ? worst : static_cast<int64_t>(cus) * 4;
+    grid = (grid + 31) / 32 * 32;  // the ring kernels deal tiles to the XCDs four at a time
+  }
+  // Dense launches of many rounds of equal tiles run one resident workgroup per CU that walks its tiles itself (the
+  // ring kernels loop over tiles anyway): saves the hardware's per-workgroup start, 4 % at six rounds.
+  r.resident = mode == kDense && grid >= 4ll * cus;
+  r.grid = grid;
+  return r;
 }
 
 struct Problem {
@@ -552,13 +620,13 @@ int run(const Problem& pr) {
   const int cus = device_cu_count(&dev);
   if (cus < 0) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
 
-  Plan pl = make_plan(pr.mode, pr.rows, pr.N, pr.K, cus, pr.ws ? pr.ws_bytes : 0);
-  if (g_knob[kKnobSplitK] > 0 && pr.mode == kDense && pl.variant != kVarExact && !is_skinny(pl.variant) &&
-      pl.variant != kVarPipe256mix)
-    pl.splitk = clamp_splitk(g_knob[kKnobSplitK], pr.rows, pr.N, static_cast<int>(kblocks) * 2,
-                             pr.ws && pr.ws_bytes > DLB_WS_COUNTER_BYTES ? pr.ws_bytes - DLB_WS_COUNTER_BYTES : 0);
   if (pr.ws && misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
-  if (pl.splitk > 1 && (!pr.ws || pr.ws_bytes <= DLB_WS_COUNTER_BYTES)) pl.splitk = 1;
+  const Resolved rs = resolve(pr.mode, pr.rows, pr.N, pr.K, pr.G, pr.as_sm, pr.as_sk, pr.ws != nullptr, pr.ws_bytes, cus);
+  const Plan& pl = rs.pl;
+  // everything that can refuse the launch is checked before the first pre-pass kernel is enqueued
+  if (rs.grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)rs.grid);
+  if (pl.variant == kVarExact && pr.mode != kDense) return fail(DLB_ERR_BAD_SHAPE, "exact path is dense only");
+  if (pl.variant == kVarExact && ceil_div(pr.N, 64) > (1ll << 31) - 1) return fail(DLB_ERR_BAD_SHAPE, "N too large for the exact path");
 
   Args ar;
   memset(&ar, 0, sizeof(ar));
@@ -584,9 +652,8 @@ int run(const Problem& pr) {
   ar.tiles_m = static_cast<int>(ceil_div(pr.rows, pl.bm));
   ar.tiles_n = static_cast<int>(ceil_div(pr.N, pl.bn));
   ar.sk_bn = pl.sk_bn;
-  ar.splitk = pl.splitk;
-  ar.kb_per_split = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, pl.splitk));
-  ar.splitk = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, ar.kb_per_split));  // no empty splits
+  ar.splitk = rs.splitk;
+  ar.kb_per_split = rs.kb_per_split;
   ar.group_m = g_knob[kKnobGroupM] > 0 ? g_knob[kKnobGroupM] : 8;
   ar.out_f32 = pr.out_dtype == DLB_OUT_F32;
   const size_t esz = ar.out_f32 ? 4 : 2;
@@ -598,93 +665,61 @@ int run(const Problem& pr) {
   }
 
   hipError_t e = hipSuccess;
-  // expert-contiguous rows: a device-built list of 256- and 128-row tiles (see contiguous_tile_list_kernel); its
-  // storage sits at the head of the workspace's data region, the re-laid scales behind it
+  // workspace data region: [tile list][re-laid scales][partial sums of the K slices]
   size_t ws_used = 0;
-  bool tile_list = false;
-  if (pr.mode == kContiguous && pl.variant == kVarPipe128x256w8 && g_forced_variant < 0 && ar.ws && kblocks > 0) {
-    const int64_t nblk = ceil_div(pr.rows, kScaleBlock);
-    const size_t bytes = (static_cast<size_t>(2 + 2 * nblk) * sizeof(int32_t) + 255) / 256 * 256;
-    if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= pr.ws_bytes) {
-      int32_t* tl = reinterpret_cast<int32_t*>(ar.ws);
-      hipLaunchKernelGGL(contiguous_tile_list_kernel, dim3(1), dim3(256), 0, pr.stream, pr.gidx, static_cast<int>(pr.rows), pr.G, tl,
-                         static_cast<int>(nblk));
-      e = hipGetLastError();
-      if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "tile list launch failed: %s", hipGetErrorString(e));
-      ar.tlist = tl;
-      ar.tlist_cap = static_cast<int>(nblk);
-      ws_used = bytes;
-      tile_list = true;
-    }
+  const bool tile_list = rs.tile_list;
+  if (tile_list) {
+    // expert-contiguous rows: a device-built list of 256- and 128-row tiles (see contiguous_tile_list_kernel)
+    int32_t* tl = reinterpret_cast<int32_t*>(ar.ws);
+    hipLaunchKernelGGL(contiguous_tile_list_kernel, dim3(1), dim3(256), 0, pr.stream, pr.gidx, static_cast<int>(pr.rows), pr.G, tl,
+                       static_cast<int>(rs.nblk));
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "tile list launch failed: %s", hipGetErrorString(e));
+    ar.tlist = tl;
+    ar.tlist_cap = static_cast<int>(rs.nblk);
+    ws_used = (static_cast<size_t>(2 + 2 * rs.nblk) * sizeof(int32_t) + 255) / 256 * 256;
   }
-  if (is_pipelined(pl.variant) && pr.as_sk == 1 && pr.as_sm > 1 && ar.ws && kblocks > 1) {
-    // row-major activation scales: re-lay them rows-contiguous in the workspace first (a few microseconds) so the
-    // GEMM fetches 8 cache lines of scales per K step and tile instead of 256
-    const int64_t rows_pad = (pr.rows + 3) / 4 * 4;
-    const int64_t need = groups * kblocks * rows_pad * static_cast<int64_t>(sizeof(float));
-    if (static_cast<size_t>(need) + ws_used + DLB_WS_COUNTER_BYTES <= pr.ws_bytes && rows_pad * kblocks < (1ll << 31)) {
-      float* relaid = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
-      const dim3 tgrid(static_cast<unsigned>(ceil_div(rows_pad, 32)), static_cast<unsigned>(ceil_div(kblocks, 32)),
-                       static_cast<unsigned>(pr.mode == kMasked ? groups : 1));
-      hipLaunchKernelGGL(fp8_scale_transpose_kernel, tgrid, dim3(256), 0, pr.stream, pr.a_s, relaid, static_cast<int>(pr.rows),
-                         static_cast<int>(kblocks), static_cast<int>(rows_pad), pr.mode == kMasked ? pr.as_sg : 0, pr.as_sm,
-                         pr.as_sk);
-      e = hipGetLastError();
-      if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "scale re-layout launch failed: %s", hipGetErrorString(e));
-      ar.a_s = relaid;
-      ar.as_sm = 1;
-      ar.as_sk = rows_pad;
-      ar.as_gs = kblocks * rows_pad;
-      ws_used += (static_cast<size_t>(need) + 255) / 256 * 256;
-    }
+  if (rs.relayout) {
+    float* relaid = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
+    const dim3 tgrid(static_cast<unsigned>(ceil_div(rs.rows_pad, 32)), static_cast<unsigned>(ceil_div(kblocks, 32)),
+                     static_cast<unsigned>(pr.mode == kMasked ? groups : 1));
+    hipLaunchKernelGGL(fp8_scale_transpose_kernel, tgrid, dim3(256), 0, pr.stream, pr.a_s, relaid, static_cast<int>(pr.rows),
+                       static_cast<int>(kblocks), static_cast<int>(rs.rows_pad), pr.mode == kMasked ? pr.as_sg : 0, pr.as_sm,
+                       pr.as_sk);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "scale re-layout launch failed: %s", hipGetErrorString(e));
+    ar.a_s = relaid;
+    ar.as_sm = 1;
+    ar.as_sk = rs.rows_pad;
+    ar.as_gs = kblocks * rs.rows_pad;
   }
-  if (ar.splitk > 1 && is_pipelined(pl.variant)) {
-    // the partial matrices of the K slices follow whatever else lives in the workspace; fewer slices if they do not fit
-    const size_t avail = pr.ws_bytes - DLB_WS_COUNTER_BYTES - ws_used;
-    const size_t per_slice = static_cast<size_t>(pr.rows) * pr.N * sizeof(float);
-    if (per_slice * ar.splitk > avail) {
-      const int s = per_slice > 0 && avail / per_slice >= 1 ? static_cast<int>(avail / per_slice) : 1;
-      ar.kb_per_split = static_cast<int>(ceil_div(kblocks, s));
-      ar.splitk = static_cast<int>(ceil_div(kblocks, ar.kb_per_split));
-    }
-    ar.ws = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
-  }
-  const int64_t tiles = static_cast<int64_t>(ar.tiles_m) * ar.tiles_n * ar.splitk;
+  if (ar.splitk > 1 && is_pipelined(pl.variant)) ar.ws = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + rs.ws_used);
   switch (pl.variant) {
     case kVarExact: {
-      if (pr.mode != kDense) return fail(DLB_ERR_BAD_SHAPE, "exact path is dense only");
-      const dim3 grid(static_cast<unsigned>(ceil_div(pr.N, 64)), static_cast<unsigned>(ceil_div(pr.rows, 4)));
+      // rows in a grid-stride loop: the second grid dimension is limited to 65535
+      const int64_t row_groups = ceil_div(pr.rows, 4);
+      const dim3 grid(static_cast<unsigned>(ceil_div(pr.N, 64)), static_cast<unsigned>(row_groups < 65535 ? row_groups : 65535));
       hipLaunchKernelGGL(fp8_gemm_exact_kernel, grid, dim3(256), 0, pr.stream, ar);
       e = hipGetLastError();
       break;
     }
     case kVarSkinny16:
-      e = launch_skinny(1, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
+      e = launch_skinny(1, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
       break;
     case kVarSkinny32:
-      e = launch_skinny(2, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
+      e = launch_skinny(2, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
       break;
     case kVarSkinny64:
-      e = launch_skinny(4, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
+      e = launch_skinny(4, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
       break;
     case kVarSkinny128:
-      e = launch_skinny(8, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, ar, dev, pr.stream);
+      e = launch_skinny(8, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
       break;
     default: {
-      int64_t grid = tiles;
-      if (pr.mode == kMasked) {
-        // the real tile count is only known on the device; cover the worst case with a resident-sized grid
-        const int64_t worst = static_cast<int64_t>(ar.tiles_m) * ar.tiles_n * pr.G;
-        grid = worst < static_cast<int64_t>(cus) * 4 ? worst : static_cast<int64_t>(cus) * 4;
-        grid = (grid + 31) / 32 * 32;  // the ring kernels deal tiles to the XCDs four at a time
-      }
-      if (grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)grid);
-      const int g = static_cast<int>(grid);
-      // Dense launches of many rounds of equal tiles run one resident workgroup per CU that walks its tiles itself
-      // (the ring kernels loop over tiles anyway): saves the hardware's per-workgroup start, 4 % at six rounds.
-      const int g_dense = pr.mode == kDense && grid >= 4ll * cus ? cus : g;
+      const int g = static_cast<int>(rs.grid);
+      const int g_dense = rs.resident ? cus : g;
       if (pl.variant == kVarPipe256mix) {
-        const int64_t split = pick_mixed_split(pr.rows, pr.N, cus);
+        const int64_t split = rs.n_split;
         if (split >= pr.N) {
           e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
         } else {
@@ -701,11 +736,7 @@ int run(const Problem& pr) {
             e = hipGetLastError();
           }
         }
-      } else if (pl.variant == kVarPipe256x128)
-        e = launch_pipelined_mode<Pipe256x128>(pr.mode, ar, g, dev, pr.stream);
-      else if (pl.variant == kVarPipe128x256)
-        e = launch_pipelined_mode<Pipe128x256>(pr.mode, ar, g, dev, pr.stream);
-      else if (pl.variant == kVarPipe256x256)
+      } else if (pl.variant == kVarPipe256x256)
         e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
       else if (pl.variant == kVarPipe128x256w8 && tile_list) {
         static std::atomic<unsigned long long> lds_done{0};
@@ -900,15 +931,20 @@ int dlb_fp8_quant_128x128(const void* w, int w_dtype, void* q, float* s, int64_t
 }
 
 int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t workspace_bytes, int compute_units, int* variant,
-                      int* k_slices, int* decode_columns) {
+                      int* k_slices, int* decode_columns, int64_t* narrow_from) {
   dlb::clear_error();
   if (mode < dlb::kDense || mode > dlb::kMasked) return dlb::fail(DLB_ERR_BAD_SHAPE, "mode %d is not 0 (dense), 1 (contiguous) or 2 (masked)", mode);
   if (rows < 0 || N < 0 || K < 0) return dlb::fail(DLB_ERR_BAD_SHAPE, "negative dimension (rows=%lld, N=%lld, K=%lld)", (long long)rows, (long long)N, (long long)K);
+  const int64_t lim = (1ll << 31) - 1024;
+  if (rows > lim || N > lim || K > lim) return dlb::fail(DLB_ERR_BAD_SHAPE, "dimension beyond 2^31");
   if (compute_units <= 0) return dlb::fail(DLB_ERR_BAD_SHAPE, "compute_units must be positive");
-  const dlb::Plan pl = dlb::make_plan(mode, rows, N, K, compute_units, workspace_bytes);
-  if (variant) *variant = pl.variant;
-  if (k_slices) *k_slices = pl.splitk;
-  if (decode_columns) *decode_columns = dlb::is_skinny(pl.variant) ? pl.sk_bn : 0;
+  // row-major activation scales, as the dense Python entry point hands them over
+  const dlb::Resolved rs = dlb::resolve(mode, rows, N, K, mode == dlb::kDense ? 1 : 32, dlb::ceil_div(K, dlb::kScaleBlock), 1,
+                                        workspace_bytes > 0, workspace_bytes, compute_units);
+  if (variant) *variant = rs.pl.variant;
+  if (k_slices) *k_slices = rs.splitk;
+  if (decode_columns) *decode_columns = dlb::is_skinny(rs.pl.variant) ? rs.pl.sk_bn : 0;
+  if (narrow_from) *narrow_from = rs.n_split;
   return DLB_OK;
 }
 

@@ -45,7 +45,7 @@
 extern "C" {
 #endif
 
-#define DLB_ABI_VERSION 1
+#define DLB_ABI_VERSION 2
 
 /* output element type of C */
 #define DLB_OUT_BF16 0
@@ -86,8 +86,9 @@ size_t dlb_fp8_gemm_workspace_bytes(int64_t rows, int64_t N, int64_t K);
  *   b_s  [ceil(N/128), ceil(K/128)] fp32, row-major
  *   c    [M, N]                     bf16 or fp32 (out_dtype), row-major, row stride N
  *
- * M, N, K >= 0 (M == 0 or N == 0 enqueues nothing; K == 0 stores zeros).  Any M, N, K are accepted;
- * K % 16 == 0 takes the MFMA path, other K a slower exact path.
+ * M, N, K >= 0 (M == 0 or N == 0 enqueues nothing; K == 0 stores zeros).  Any M, N, K below 2^31 - 1024 are accepted;
+ * K % 16 == 0 takes the MFMA path, other K a slower exact path.  K >= 2^24 (or an a_s row stride >= 2^21 floats) is
+ * beyond the 32-bit offsets of the DMA kernels and runs on the register-staged kernels instead.
  */
 int dlb_fp8_gemm(const void* a, const void* b, const float* a_s, const float* b_s, void* c,
                  int64_t M, int64_t N, int64_t K,
@@ -204,13 +205,16 @@ int dlb_fp8_quant_128x128(const void* w, int w_dtype, void* q, float* s, int64_t
 /*
  * Host-only query: what the library would launch for a problem, without launching anything (no GPU is touched).
  * mode 0 = dlb_fp8_gemm, 1 = grouped contiguous (rows = M_sum), 2 = grouped masked (rows = M_max); `compute_units`
- * is the CU count to plan for (256 on MI355X).  Outputs (each may be NULL): the kernel variant id
- * (dlb_fp8_gemm_variant_name), the number of K slices summed in a second pass (1 = none), the output columns per
- * workgroup of the decode kernels (0 for other variants).  Honours the calling thread's forced variant and knobs, as
- * a launch would.  No counterpart in the reference, whose single Triton configuration needs no plan.
+ * is the CU count to plan for (256 on MI355X); activation scales are taken to be row-major.  Outputs (each may be
+ * NULL): the kernel variant id (dlb_fp8_gemm_variant_name); the number of K slices summed in a second pass (1 = none),
+ * exactly as a launch with this workspace size would use it; the output columns per workgroup of the decode kernels
+ * (0 for other variants); the first column of the 192-wide tiles of the mixed-width prefill launch (N when all tiles
+ * are equal).  Honours the calling thread's forced variant and knobs, as a launch does (both run the same code).
+ * Costs a few microseconds at most and keeps no state.  No counterpart in the reference, whose single Triton
+ * configuration needs no plan.
  */
 int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t workspace_bytes, int compute_units, int* variant,
-                      int* k_slices, int* decode_columns);
+                      int* k_slices, int* decode_columns, int64_t* narrow_from);
 
 /*
  * Tuning / test hook: force the kernel variant the next calls FROM THIS THREAD use.

@@ -7,7 +7,7 @@ import pytest
 from dlblas_amd import _lib
 
 DENSE, CONTIGUOUS, MASKED = 0, 1, 2
-RING = ('pipe256x128', 'pipe128x256', 'pipe256x256', 'pipe128x256w8', 'pipe256mix', 'pipe128x128', 'pipe128x64')
+RING = ('pipe256x256', 'pipe128x256w8', 'pipe256mix', 'pipe128x128', 'pipe128x64')
 DECODE = {'skinny16': 16, 'skinny32': 32, 'skinny64': 64, 'skinny128': 128}
 
 
@@ -78,7 +78,103 @@ def test_plan_follows_the_hooks_and_rejects_nonsense():
         _lib.force_variant(None)
         _lib.tune('splitk', 0)
     lib = _lib.load()
-    assert lib.dlb_fp8_gemm_plan(7, 1, 1, 1, 0, 256, None, None, None) == _lib.ERR_BAD_SHAPE
-    assert lib.dlb_fp8_gemm_plan(0, -1, 1, 1, 0, 256, None, None, None) == _lib.ERR_BAD_SHAPE
-    assert lib.dlb_fp8_gemm_plan(0, 1, 1, 1, 0, 0, None, None, None) == _lib.ERR_BAD_SHAPE
-    assert lib.dlb_fp8_gemm_plan(0, 16, 7168, 2048, 0, 256, None, None, None) == 0
+    assert lib.dlb_fp8_gemm_plan(7, 1, 1, 1, 0, 256, None, None, None, None) == _lib.ERR_BAD_SHAPE
+    assert lib.dlb_fp8_gemm_plan(0, -1, 1, 1, 0, 256, None, None, None, None) == _lib.ERR_BAD_SHAPE
+    assert lib.dlb_fp8_gemm_plan(0, 1, 1, 1, 0, 0, None, None, None, None) == _lib.ERR_BAD_SHAPE
+    assert lib.dlb_fp8_gemm_plan(0, 16, 7168, 2048, 0, 256, None, None, None, None) == 0
+
+
+def test_k_slices_are_what_a_launch_uses():
+    """The plan query runs the code a launch runs: the slice-count knob, the no-empty-slice rule and the workspace
+    clamp all show in its answer."""
+    try:
+        for want in (2, 3, 5, 7, 16):
+            _lib.tune('splitk', want)
+            v, s, _ = _lib.plan(DENSE, 200, 392, 2048)                       # 16 K blocks
+            per = -(-16 // min(want, 16))
+            assert s == -(-16 // per), (want, v, s)                          # slices of `per` blocks, none empty
+            assert _lib.plan(DENSE, 200, 392, 2048, workspace_bytes=0)[1] == 1
+            # a workspace that holds exactly two partial matrices (plus the re-laid scales of the ring kernels)
+            tight = _lib.WS_COUNTER_BYTES + 2 * 200 * 392 * 4 + 16 * 200 * 4 + 512
+            assert _lib.plan(DENSE, 200, 392, 2048, workspace_bytes=tight)[1] <= 2
+        _lib.tune('splitk', 0)
+        _lib.force_variant('pipe256mix')
+        _lib.tune('splitk', 4)
+        assert _lib.plan(DENSE, 4096, 7168, 2048)[1] == 1                    # the mixed-width launch never splits K
+    finally:
+        _lib.tune('splitk', 0)
+        _lib.force_variant(None)
+
+
+def test_mixed_width_split_matches_a_tile_by_tile_simulation():
+    """The closed-form makespan behind the choice of the narrow-tile region against the obvious simulation: tiles handed
+    out one by one to the worker that is free first."""
+    import heapq
+
+    def makespan(ta, tb, cb, workers):
+        free = [0.0] * workers
+        end = 0.0
+        for t in range(ta + tb):
+            done = heapq.heappop(free) + (1.0 if t < ta else cb)
+            heapq.heappush(free, done)
+            end = max(end, done)
+        return end
+
+    def pick(M, N, cus):
+        tm = -(-M // 256)
+        if tm * -(-N // 256) > 16 * cus:
+            return N
+        uniform = makespan(tm * -(-N // 256), 0, 0.78, cus)
+        best, best_split = uniform, N
+        for ca in range(N // 256, -1, -1):
+            split = ca * 256
+            if split >= N:
+                continue
+            t = makespan(tm * ca, tm * -(-(N - split) // 192), 0.78, cus)
+            if t < best - 1e-6 and t < 0.96 * uniform:
+                best, best_split = t, split
+        return best_split
+
+    _lib.force_variant('pipe256mix')
+    try:
+        for M, N, cus in [(4096, 7168, 256), (4096, 24576, 256), (2048, 7168, 256), (4096, 4096, 256), (1024, 2112, 80),
+                          (300, 7168, 64), (8192, 1536, 256), (4000, 5000, 304), (512, 16384, 256), (256, 256, 256)]:
+            assert _lib.plan_full(DENSE, M, N, 2048, compute_units=cus)[3] == pick(M, N, cus), (M, N, cus)
+    finally:
+        _lib.force_variant(None)
+    assert _lib.plan_full(DENSE, 4096, 7168, 18432) == ('pipe256mix', 1, 0, 4096)
+    assert _lib.plan_full(DENSE, 16, 7168, 2048)[3] == 7168
+
+
+def test_planning_a_thousand_prefill_shapes_is_cheap():
+    """A serving loop sees a new M with almost every prefill request: the planner keeps no per-shape state and has to
+    answer in microseconds.  1000 distinct (M, N), each planned once; 20 us per plan on average including the ctypes
+    call."""
+    import time
+    shapes = [(257 + 37 * i, (1536, 2112, 4096, 7168, 18432, 24576)[i % 6] + 128 * (i % 7)) for i in range(1000)]
+    assert len(set(shapes)) == 1000
+    _lib.plan(DENSE, 4096, 7168, 18432)
+    t0 = time.perf_counter()
+    for M, N in shapes:
+        _lib.plan(DENSE, M, N, 7168)
+    per_plan = (time.perf_counter() - t0) / len(shapes)
+    assert per_plan < 20e-6, f'{per_plan * 1e6:.1f} us per plan'
+
+
+def test_shapes_beyond_32_bit_dma_offsets_take_the_64_bit_kernels():
+    assert _lib.plan(DENSE, 4096, 4096, 1 << 24)[0] == 'tile128x128'
+    assert _lib.plan(DENSE, 4096, 4096, (1 << 24) - 128)[0] in RING
+    assert _lib.plan(CONTIGUOUS, 1024, 4096, 1 << 24)[0] == 'tile128x128'
+    assert _lib.plan(DENSE, 16, 4096, 1 << 24)[0] == 'skinny16'              # its register-load form: 64-bit addressing
+    lib = _lib.load()
+    assert lib.dlb_fp8_gemm_plan(0, 1 << 31, 1, 1, 0, 256, None, None, None, None) == _lib.ERR_BAD_SHAPE
+
+
+def test_decode_wave_count_is_clamped_to_the_lds():
+    """16 waves x 16 fragments would need 256 KB for the partial sums of a 128-row decode launch: the knob is honoured
+    only as far as the 160 KB of LDS allow (the launch itself is exercised on the GPU)."""
+    try:
+        _lib.tune('skinny_waves', 16)
+        assert _lib.plan(DENSE, 128, 7168, 2048)[0] == 'skinny128'
+    finally:
+        _lib.tune('skinny_waves', 0)
