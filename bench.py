@@ -113,12 +113,9 @@ class DenseLauncher:
             _lib.check(rc)
 
 
-def time_steps(launch, steps, warmup):
-    """Wall clock over exactly `steps` launches between two synchronisations, plus the HIP-event time of the same
-    launches on the launch stream (average kernel duration when launches are back to back)."""
+def _timed(launch, steps):
+    """Wall clock and HIP-event time (events on the launch stream) of exactly `steps` back-to-back launches."""
     import torch
-    for _ in range(warmup):
-        launch()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -129,6 +126,51 @@ def time_steps(launch, steps, warmup):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     return wall_ms / steps, start.elapsed_time(stop) / steps
+
+
+SETTLE_MAX_LAUNCHES = 120
+
+
+def settle(launch, block=10, tol=0.01):
+    """Untimed launches of the step until the power controller has settled: a GPU that goes from idle to this load
+    boosts, overshoots into a throttle and recovers over the first few tens of milliseconds (per-launch series in
+    profiles/).  Blocks of `block` launches are timed until two consecutive blocks agree within `tol`, at most
+    SETTLE_MAX_LAUNCHES launches.  Returns the number of launches made."""
+    import torch
+    done, prev = 0, None
+    while done < SETTLE_MAX_LAUNCHES:
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(block):
+            launch()
+        stop.record()
+        torch.cuda.synchronize()
+        done += block
+        cur = start.elapsed_time(stop)
+        if prev is not None and abs(cur - prev) <= tol * prev:
+            break
+        prev = cur
+    return done
+
+
+def time_steps(launch, steps, warmup):
+    """The measurement of the headline workload.
+
+    1. From an idle GPU: `warmup` untimed + `steps` timed launches.  Reported as "from_idle": on this part it is the
+       power controller's start-up transient, not the kernel's rate.
+    2. settle(): untimed launches until the per-launch time stops moving.
+    3. `warmup` untimed launches, then EXACTLY `steps` timed launches between two synchronisations: wall clock
+       (ms_per_step, value) and HIP events on the launch stream (roofline)."""
+    import torch
+    time.sleep(0.2)
+    for _ in range(warmup):
+        launch()
+    idle_wall, idle_ev = _timed(launch, steps)
+    settled = settle(launch)
+    for _ in range(warmup):
+        launch()
+    wall, ev = _timed(launch, steps)
+    return wall, ev, {'ms_per_step': idle_wall, 'kernel_ms': idle_ev, 'settle_launches': settled}
 
 
 def cpu_baseline(kind, M, N, K, a_q, a_s, b_q, b_s, budget_s=12.0):
@@ -185,13 +227,52 @@ def decode_sweep(dev):
     for (M, N, K) in DECODE_SWEEP:
         a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=24)
         out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-        ms = time_call(DenseLauncher(a_q, a_s, ws, out), 480, 48)
+        ms = time_call(DenseLauncher(a_q, a_s, ws, out), 480, 1500)  # 1500 untimed launches (~10 ms): clocks at their loaded level
         nbytes = algorithmic_bytes(M, N, K)
         rows.append({'workload': f'decode_{M}x{N}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
                      'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'TFLOPs': 2.0 * M * N * K / ms / 1e9,
                      'bytes': nbytes})
         del a_q, a_s, ws, out
     return rows
+
+
+FLOOR_LIB = os.path.join(ROOT, 'bench_kernels', 'libfloor_kernels.so')
+
+
+def decode_floor(dev, N=7168, K=2048, copies=24):
+    """What one launch of the decode shape costs on this GPU without any arithmetic (bench_kernels/floor_kernels.hip):
+    an empty kernel of the decode kernel's grid, and a kernel that only reads the N x K weight bytes with 16-byte loads,
+    both launched back to back on one stream over the same rotation of `copies` weight buffers as the decode sweep."""
+    import torch
+    if not os.path.exists(FLOOR_LIB):
+        return None
+    lib = ctypes.CDLL(FLOOR_LIB)
+    lib.floor_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
+    lib.floor_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    bufs = [torch.randint(0, 255, (N * K, ), dtype=torch.uint8, device=dev) for _ in range(copies)]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    state = {'i': 0}
+
+    def reader(wgs, depth):
+        def read():
+            b = bufs[state['i']]
+            state['i'] = (state['i'] + 1) % copies
+            lib.floor_read(ctypes.c_void_p(b.data_ptr()), N * K, wgs, depth, stream)
+        return read
+
+    empty_ms = time_call(lambda: lib.floor_empty(cus, stream), 480, 1500)
+    # the best of a few shapes of the read-only kernel: workgroups per CU x 16-byte loads in flight per thread
+    tried = {}
+    for per_cu in (1, 2, 4):
+        for depth in (2, 4, 8):
+            tried[f'{per_cu} wg/cu x {depth} loads'] = time_call(reader(cus * per_cu, depth), 240, 240) * 1e3
+    best = min(tried, key=tried.get)
+    read_us = time_call(reader(cus * int(best.split()[0]), int(best.split()[3])), 480, 1500) * 1e3
+    return {'empty_launch_us': empty_ms * 1e3, 'read_only_us': read_us, 'read_only_GBps': N * K / read_us / 1e3,
+            'read_only_shape': best, 'bytes_read': N * K,
+            'note': 'bench-only kernels (bench_kernels/floor_kernels.hip), same rotation of weight buffers and same launch '
+                    'loop as the decode rows; read_only = fastest of 9 shapes of a kernel that only loads the weight bytes'}
 
 
 def second_prefill_workload(dev):
@@ -201,7 +282,7 @@ def second_prefill_workload(dev):
     M, N, K = 4096, 24576, 1536
     a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=1)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-    ms = time_call(DenseLauncher(a_q, a_s, ws, out), 30, 5)
+    ms = time_call(DenseLauncher(a_q, a_s, ws, out), 60, 150)  # past the power controller's start-up transient
     flops, nbytes = 2.0 * M * N * K, algorithmic_bytes(M, N, K)
     return [{'workload': f'prefill_{M}x{N}x{K}', 'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9,
              'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS, 'GBps': nbytes / ms / 1e6,
@@ -255,7 +336,7 @@ def grouped_workloads(dev):
     a_q, a_s = quantise_act(torch.randn(M_sum, K, device=dev, generator=gd).to(torch.bfloat16))
     w_q, w_s = expert_weights(G, N, K, dev, 22)
     out = torch.empty(M_sum, N, dtype=torch.bfloat16, device=dev)
-    ms = time_call(lambda: fp8_gemm_grouped_contiguous(a_q, a_s, w_q, w_s, out, m_indices), 20, 3)
+    ms = time_call(lambda: fp8_gemm_grouped_contiguous(a_q, a_s, w_q, w_s, out, m_indices), 40, 80)
     flops = 2.0 * c['tokens'] * N * K
     nbytes = M_sum * K + G * N * K + 4 * M_sum * (K // 128) + 4 * G * (N // 128) * (K // 128) + 2 * M_sum * N + 4 * M_sum
     rows.append({'workload': f'grouped_contiguous_E{G}_T{c["tokens"]}_N{N}_K{K}', 'M_sum_padded': M_sum,
@@ -272,7 +353,7 @@ def grouped_workloads(dev):
     out = torch.empty(G, M_max, N, dtype=torch.bfloat16, device=dev)
     mm = masked_m.to(dev)
     hint = int(masked_m.float().mean())
-    ms = time_call(lambda: fp8_gemm_grouped_masked(a_q, a_s, w_q, w_s, out, mm, hint), 20, 3)
+    ms = time_call(lambda: fp8_gemm_grouped_masked(a_q, a_s, w_q, w_s, out, mm, hint), 60, 150)
     valid = int(masked_m.sum())
     flops = 2.0 * valid * N * K
     nbytes = valid * K + G * N * K + 4 * valid * (K // 128) + 4 * G * (N // 128) * (K // 128) + 2 * valid * N + 4 * G
@@ -425,6 +506,8 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run three 1 GiB device copies: the known-size kernel that HBM counters are scaled by')
     ap.add_argument('--no-other', action='store_true', help='skip the decode sweep and the grouped workloads')
+    ap.add_argument('--decode-floor', action='store_true',
+                    help='run only the launch-cost floors of the decode shape (empty kernel, read-only kernel) and print them')
     ap.add_argument('--grouped-only', action='store_true',
                     help='run only the two grouped MoE workloads and print their rows (the command the rocprofv3 summaries of '
                     'the grouped kernels are made with)')
@@ -443,6 +526,10 @@ def main():
     if args.variant:
         _lib.force_variant(args.variant)
 
+    if args.decode_floor:
+        print(json.dumps({'decode_floor': decode_floor(dev)}), flush=True)
+        return
+
     if args.grouped_only:
         rows = grouped_workloads(dev)
         if args.copy_calibration:
@@ -458,7 +545,7 @@ def main():
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     launch = DenseLauncher(a_q, a_s, weights, out)
     log('timing')
-    ms_per_step, ev_ms = time_steps(launch, args.steps, args.warmup)
+    ms_per_step, ev_ms, from_idle = time_steps(launch, args.steps, args.warmup)
     flops = 2.0 * M * N * K
     nbytes = algorithmic_bytes(M, N, K)
     if memory_bound:
@@ -471,6 +558,10 @@ def main():
     roofline['frac'] = roofline['achieved'] / roofline['peak']
     roofline['traffic'] = measured_traffic(args.workload)
     roofline['kernel_ms'] = ev_ms
+    from_idle['frac_of_peak'] = (nbytes / 1e9 if memory_bound else flops / 1e12) / (from_idle['kernel_ms'] * 1e-3) / roofline['peak']
+    from_idle['note'] = ('the same warmup + steps measured first, on an idle GPU: the power controller boosts, throttles and '
+                         'recovers during the first tens of milliseconds of this load; value / roofline are measured after '
+                         'settle_launches further untimed launches, when the per-launch time has stopped moving')
 
     result = {
         'metric': 'FP8 block-scaled GEMM TFLOP/s (% FP8 MFMA peak); decode-M HBM GB/s',
@@ -488,6 +579,7 @@ def main():
         'config': {'workload': args.workload, 'M': M, 'N': N, 'K': K, 'a_scale': '1x128 f32', 'b_scale': '128x128 f32',
                    'out': 'bf16', 'seed': 20},
         'roofline': roofline,
+        'from_idle': from_idle,
     }
 
     if not args.no_other:
@@ -496,6 +588,7 @@ def main():
         m16 = next(r for r in others if r['workload'] == 'decode_16x7168x2048')
         result['decode'] = {'workload': m16['workload'], 'us_per_launch': m16['us_per_launch'], 'GBps': m16['GBps'],
                             'frac_of_hbm_peak': m16['frac_of_hbm_peak'], 'bytes': m16['bytes'],
+                            'floor_us': decode_floor(dev),
                             'note': '24 distinct weight copies in rotation (353 MB) so reads miss the 256 MB cache'}
         log('grouped workloads')
         others += second_prefill_workload(dev)

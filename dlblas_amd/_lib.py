@@ -136,15 +136,22 @@ def prepare(device=None, stream=None) -> None:
         st.synchronize()
 
 
+_variant_names = None
+
+
 def variant_names():
-    lib = load()
-    names, i = [], 0
-    while True:
-        name = lib.dlb_fp8_gemm_variant_name(i)
-        if name is None:
-            return names
-        names.append(name.decode())
-        i += 1
+    global _variant_names
+    if _variant_names is None:
+        lib = load()
+        names, i = [], 0
+        while True:
+            name = lib.dlb_fp8_gemm_variant_name(i)
+            if name is None:
+                break
+            names.append(name.decode())
+            i += 1
+        _variant_names = names
+    return list(_variant_names)
 
 
 def plan(mode: int, rows: int, N: int, K: int, workspace_bytes: int = None, compute_units: int = 256):
