@@ -29,6 +29,8 @@ WORKLOADS = {
     'prefill_4096x24576x1536': ('dense', 4096, 24576, 1536),
     'decode_16x7168x2048': ('dense', 16, 7168, 2048),
     'decode_16x2112x7168': ('dense', 16, 2112, 7168),
+    'decode_64x2112x7168': ('dense', 64, 2112, 7168),
+    'decode_128x2112x7168': ('dense', 128, 2112, 7168),
     'cpu_case_64x512x1024': ('dense', 64, 512, 1024),
 }
 # measured after the timed region and reported under "other_workloads" (name: M, N, K)
@@ -506,6 +508,12 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run three 1 GiB device copies: the known-size kernel that HBM counters are scaled by')
     ap.add_argument('--no-other', action='store_true', help='skip the decode sweep and the grouped workloads')
+    ap.add_argument('--moe-only', action='store_true',
+                    help='run only the quantisers, the activation step and ep_scatter / ep_gather and print their rows (the '
+                    'command their rocprofv3 summaries are made with)')
+    ap.add_argument('--series', type=int, default=0,
+                    help='print the duration of each of the first N launches of the workload from an idle GPU (the power '
+                    "controller's start-up transient) and exit")
     ap.add_argument('--decode-floor', action='store_true',
                     help='run only the launch-cost floors of the decode shape (empty kernel, read-only kernel) and print them')
     ap.add_argument('--grouped-only', action='store_true',
@@ -530,6 +538,13 @@ def main():
         print(json.dumps({'decode_floor': decode_floor(dev)}), flush=True)
         return
 
+    if args.moe_only:
+        rows = quantiser_workload(dev) + activation_workloads(dev) + permutation_workloads(dev)
+        if args.copy_calibration:
+            copy_calibration(dev)
+        print(json.dumps({'moe_workloads': rows}), flush=True)
+        return
+
     if args.grouped_only:
         rows = grouped_workloads(dev)
         if args.copy_calibration:
@@ -544,6 +559,17 @@ def main():
     a_q, a_s, weights = make_inputs(M, N, K, dev, weight_copies=copies)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     launch = DenseLauncher(a_q, a_s, weights, out)
+    if args.series > 0:
+        time.sleep(0.2)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.series + 1)]
+        ev[0].record()
+        for i in range(args.series):
+            launch()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        us = [round(ev[i].elapsed_time(ev[i + 1]) * 1e3, 1) for i in range(args.series)]
+        print(json.dumps({'workload': args.workload, 'us_per_launch_in_order': us}), flush=True)
+        return
     log('timing')
     ms_per_step, ev_ms, from_idle = time_steps(launch, args.steps, args.warmup)
     flops = 2.0 * M * N * K

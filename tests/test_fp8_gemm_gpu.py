@@ -383,3 +383,31 @@ def test_registry_selects_and_caches_on_gpu(dev):
         torch.set_default_dtype(prev)
     ref = orc.dequant_ref(a_q.cpu(), a_s.cpu(), b_q.cpu(), b_s.cpu())
     helpers.tolerance_check(out, ref, 'registry')
+
+
+def test_registry_chooses_between_two_real_implementations(dev):
+    """'fp8_gemm' has two registered implementations (the planner's kernels, the register-staged tile kernels): both
+    match, both are benchmarked on the caller's tensors, the faster one is cached and returned, and both are right."""
+    print('case registry selection', flush=True)
+    from dlblas_amd import get_op
+    from dlblas_amd.op_registry import op_registry
+    from dlblas_amd.op_struct import match
+    for (M, N, K) in ((16, 2112, 2048), (512, 1024, 2048)):
+        a_q, a_s, b_q, b_s = (t.to(dev) for t in helpers.make_dense(M, N, K, seed=9))
+        args = (a_q, b_q, a_s, b_s)
+        cands = [impl for impl in op_registry.ops['fp8_gemm'] if match(args, impl.params)]
+        assert len(cands) == 2 and cands[0].call is not cands[1].call
+        ref = orc.dequant_ref(a_q.cpu(), a_s.cpu(), b_q.cpu(), b_s.cpu())
+        prev = torch.get_default_dtype()
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            op = get_op('fp8_gemm', args)
+            assert op in cands and get_op('fp8_gemm', args) is op
+            times = [min(impl.bench(*args) for _ in range(3)) for impl in cands]
+            other = cands[1 - cands.index(op)]
+            # the cached choice is the faster one (25 % slack: the two benches ran at different moments)
+            assert times[cands.index(op)] <= 1.25 * times[cands.index(other)], (M, N, K, times)
+            for impl in cands:
+                helpers.tolerance_check(impl(*args), ref, f'registry candidate {impl.call.__name__} {M}x{N}x{K}')
+        finally:
+            torch.set_default_dtype(prev)

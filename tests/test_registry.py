@@ -22,7 +22,9 @@ def test_fp8_ops_are_registered_at_import():
     names = get_list_op_names()
     for name in ('fp8_gemm', 'fp8_gemm_grouped_contiguous', 'fp8_gemm_grouped_masked', 'per_token_group_quant_fp8'):
         assert name in names
-    (params, ) = get_args_from_op_name('fp8_gemm')
+    both = get_args_from_op_name('fp8_gemm')   # two implementations under one name, identical parameter lists
+    assert len(both) == 2 and both[0] == both[1]
+    params = both[0]
     assert params.n_args == 4 and params.args_types == ['tensor'] * 4
     assert [a.dtype for a in params.args] == [torch.float8_e4m3fn] * 2 + [torch.float32] * 2
     assert all(a.device == 'cuda' for a in params.args)
