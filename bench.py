@@ -277,6 +277,47 @@ def decode_floor(dev, N=7168, K=2048, copies=24):
                     'loop as the decode rows; read_only = fastest of 9 shapes of a kernel that only loads the weight bytes'}
 
 
+def ceilings(dev):
+    """What the GPU gives the prefill kernel's instruction mix and the grouped kernels' weight stream with everything
+    else taken away (bench_kernels/floor_kernels.hip), measured like the workloads: launches back to back on one stream,
+    timed after ~100 ms of the same load so that clocks are at their loaded level."""
+    import torch
+    if not os.path.exists(FLOOR_LIB):
+        return None
+    lib = ctypes.CDLL(FLOOR_LIB)
+    lib.floor_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.floor_panel_stream.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    g = torch.Generator().manual_seed(20)
+    codes = torch.randint(0, 256, (12288, ), generator=g, dtype=torch.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x30                       # no NaN codes
+    operands = {'constant 1.0': torch.full((12288, ), 0x38, dtype=torch.uint8).to(dev), 'random e4m3 codes': codes.to(dev)}
+    sink = torch.empty(cus * 512, dtype=torch.float32, device=dev)
+    iters = 400                                                 # ~1 ms per launch
+    flop = cus * 8.0 * iters * 16 * 131072
+    res = {'mfma_loop_TFLOPs': {}, 'panel_stream_GBps': {}}
+    for name, buf in operands.items():
+        for reads in (0, 3):
+            def run(buf=buf, reads=reads):
+                lib.floor_mfma(ctypes.c_void_p(buf.data_ptr()), ctypes.c_void_p(sink.data_ptr()), cus, iters, reads, stream)
+            ms = time_call(run, 40, 100)
+            res['mfma_loop_TFLOPs'][f'{name}, {reads} ds_read_b128 per MFMA pair'] = flop / ms / 1e9
+    # 256-row panels of a [65536, 7168]-byte matrix (470 MB: past the 256 MB cache), the rows of one expert's weight tile
+    panels, row_bytes = 256, 7168
+    mat = torch.randint(0, 255, (panels * 256 * row_bytes, ), dtype=torch.uint8, device=dev)
+    for depth in (1, 2, 4):
+        def run(depth=depth):
+            lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, cus, depth, stream)
+        ms = time_call(run, 20, 20)
+        res['panel_stream_GBps'][f'{depth} K steps (x 32 KB) in flight per workgroup'] = panels * 256 * row_bytes / ms / 1e6
+    res['note'] = ('mfma_loop: pairs of v_mfma_f32_32x32x64_f8f6f4 + 16 scale FMAs from registers, 8 waves per CU, no memory '
+                   'traffic except the optional LDS reads (the prefill kernel issues 3 per pair); peak 5000 TFLOP/s. '
+                   'panel_stream: one workgroup per CU pulls 256 x 7168-byte panels from HBM through the LDS DMA path, '
+                   '128 bytes per row and K step, and computes nothing')
+    return res
+
+
 def second_prefill_workload(dev):
     """The other prefill shape of the metric's configuration: 4096 x 24576 x 1536, where the 201 MB of bf16 output are
     most of the bytes."""
@@ -516,6 +557,9 @@ def main():
                     "controller's start-up transient) and exit")
     ap.add_argument('--decode-floor', action='store_true',
                     help='run only the launch-cost floors of the decode shape (empty kernel, read-only kernel) and print them')
+    ap.add_argument('--ceilings', action='store_true',
+                    help='print what bench-only kernels reach on this GPU: the prefill kernel\'s MFMA + FMA mix from registers '
+                         '(constant and random operands, with and without LDS reads) and a bare weight-panel stream through the LDS DMA path')
     ap.add_argument('--grouped-only', action='store_true',
                     help='run only the two grouped MoE workloads and print their rows (the command the rocprofv3 summaries of '
                     'the grouped kernels are made with)')
@@ -536,6 +580,10 @@ def main():
 
     if args.decode_floor:
         print(json.dumps({'decode_floor': decode_floor(dev)}), flush=True)
+        return
+
+    if args.ceilings:
+        print(json.dumps({'ceilings': ceilings(dev)}), flush=True)
         return
 
     if args.moe_only:

@@ -1,13 +1,24 @@
-// Bench-only kernels (not part of the library): what a launch of the decode GEMM's shape costs on this GPU when it
-// computes nothing.  bench.py times them back to back on the same rotating weight buffers as the decode workloads:
+// Bench-only kernels (not part of the library): what this GPU allows the GEMM kernels' instruction mix and access
+// patterns when everything else is taken away.  bench.py times them (--decode-floor, --ceilings):
 //   floor_empty  a kernel with the decode kernel's grid and block that returns at once: the per-launch cost of the
 //                queue (dependent launches on one stream)
 //   floor_read   every byte of the weight matrix read once with 16-byte loads, nothing else: launch cost + the time the
 //                memory system needs to deliver the bytes to 256 workgroups
+//   floor_mfma   the prefill kernel's arithmetic from registers only: pairs of v_mfma_f32_32x32x64_f8f6f4 (first of a
+//                pair on a zero accumulator) + 16 scale FMAs per pair, two waves per SIMD, optionally with the kernel's
+//                rate of LDS fragment reads (3 ds_read_b128 per pair) whose data nobody waits for.  The operands come
+//                from the caller, so the same loop runs on constant and on random e4m3 codes
+//   floor_panel_stream  one workgroup per CU streams 256-row panels of a row-major byte matrix through the LDS DMA path
+//                (global_load_lds_dwordx4, 8 rows x 128 bytes per wave instruction, K step by K step, S steps in
+//                flight) and does nothing with them: the rate at which a CU can pull a weight tile's rows from HBM
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
 __global__ void __launch_bounds__(512) floor_empty_kernel(int* sink) {
   if (sink == reinterpret_cast<int*>(1)) *sink = 0;  // never true: keeps the argument alive
@@ -31,6 +42,70 @@ __global__ void __launch_bounds__(512) floor_read_kernel(const v4i* src, int64_t
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5a5a5a5a && sink == reinterpret_cast<int*>(1)) *sink = acc.x;
 }
 
+// R = ds_read_b128 per MFMA pair (0 or 3).  in: 6 x 64 x 32 bytes of e4m3 codes (4 "A" + 2 "B" operand registers per lane).
+template <int R>
+__global__ void __launch_bounds__(512) floor_mfma_kernel(const v8i* in, float* out, int iters, float scale) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<int*>(lds)[i] = 0x38383838;
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row = lane & 31, half = lane >> 5, swz = (row & 7) ^ ((row >> 3) & 1);
+  int addr[3];
+  for (int i = 0; i < 3; ++i) addr[i] = wave * 8192 + row * 128 + ((((i >> 1) * 4 + 2 * half + (i & 1)) ^ swz) << 4);
+  v8i a[4], b[2];
+  for (int i = 0; i < 4; ++i) a[i] = in[lane + 64 * i];
+  for (int i = 0; i < 2; ++i) b[i] = in[lane + 64 * (4 + i)];
+  v16f acc[4], part[2];
+  for (int j = 0; j < 16; ++j) acc[0][j] = acc[1][j] = acc[2][j] = acc[3][j] = part[0][j] = part[1][j] = 0.0f;
+  v4i d[3] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      if (t == 4) asm volatile("" : "+v"(a[0][0]), "+v"(a[1][0]), "+v"(a[2][0]), "+v"(a[3][0]));  // pairs 4..7 are not copies of 0..3
+      __builtin_amdgcn_sched_barrier(0);
+      v16f z;
+      for (int j = 0; j < 16; ++j) z[j] = 0.0f;
+      z = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[t & 3], b[0], z, 0, 0, 0, 0, 0, 0);
+      part[t & 1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[(t + 1) & 3], b[1], z, 0, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < R; ++r) asm volatile("ds_read_b128 %0, %1" : "=v"(d[r]) : "v"(addr[r] + (t & 1) * 4096));
+      __builtin_amdgcn_sched_barrier(0);
+      acc[(t + 3) & 3] += part[(t + 1) & 1] * scale;  // the scale FMAs of the previous pair
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // fold the (constant) LDS data in and move the operands a little, so that no iteration is a copy of another
+    a[0][0] ^= it ^ (d[0].x ^ d[1].y ^ d[2].z ^ 0x38383838 ^ (R == 0 ? 0x38383838 : 0));
+    b[0][1] += 0x01010101;
+  }
+  float r = 0.0f;
+  for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 16; ++j) r += acc[i][j];
+  out[blockIdx.x * 512 + threadIdx.x] = r;
+}
+
+// S = K steps a wave keeps in flight.  Matrix [panels * 256][row_bytes]; workgroup b takes panels b, b + grid, ...
+template <int S>
+__global__ void __launch_bounds__(512) floor_panel_stream_kernel(const char* src, int panels, int64_t row_bytes) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ksteps = static_cast<int>(row_bytes / 128);
+  for (int p = blockIdx.x; p < panels; p += gridDim.x) {
+    // lane -> (row of the wave's 32, 16-byte chunk of the row's 128-byte line)
+    const char* base = src + (static_cast<int64_t>(p) * 256 + wave * 32 + (lane >> 3)) * row_bytes + (lane & 7) * 16;
+    for (int k = 0; k < ksteps; ++k) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(base + static_cast<int64_t>(u) * 8 * row_bytes + k * 128),
+                                         (lds_ptr_t)(lds + ((k % S) * 32 + wave * 4 + u) * 1024), 16, 0, 0);
+      if (S == 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (S == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      if (S == 4) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 extern "C" {
 
 int floor_empty(int workgroups, void* stream) {
@@ -49,6 +124,36 @@ int floor_read(const void* src, int64_t bytes, int workgroups, int loads_in_flig
     hipLaunchKernelGGL(floor_read_kernel<4>, grid, block, 0, st, p, bytes / 16, nullptr);
   else
     hipLaunchKernelGGL(floor_read_kernel<2>, grid, block, 0, st, p, bytes / 16, nullptr);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// operands: 12288 bytes of e4m3 codes on the device; out: workgroups * 512 floats.  FLOP per launch =
+// workgroups * 8 waves * iters * 16 MFMAs * 131072.
+int floor_mfma(const void* operands, float* out, int workgroups, int iters, int lds_reads, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const v8i* in = static_cast<const v8i*>(operands);
+  hipFuncSetAttribute(reinterpret_cast<const void*>(floor_mfma_kernel<3>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+  hipFuncSetAttribute(reinterpret_cast<const void*>(floor_mfma_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+  if (lds_reads > 0)
+    hipLaunchKernelGGL(floor_mfma_kernel<3>, dim3(workgroups), dim3(512), 65536, st, in, out, iters, 1.5f);
+  else
+    hipLaunchKernelGGL(floor_mfma_kernel<0>, dim3(workgroups), dim3(512), 65536, st, in, out, iters, 1.5f);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// src: [panels * 256][row_bytes] bytes, row_bytes a multiple of 128; steps_in_flight 1, 2 or 4
+int floor_panel_stream(const void* src, int panels, int64_t row_bytes, int workgroups, int steps_in_flight, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const char* p = static_cast<const char*>(src);
+  if (row_bytes <= 0 || row_bytes % 128 != 0 || panels <= 0) return -1;
+  const dim3 grid(workgroups), block(512);
+  hipFuncSetAttribute(reinterpret_cast<const void*>(floor_panel_stream_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
+  if (steps_in_flight >= 4)
+    hipLaunchKernelGGL(floor_panel_stream_kernel<4>, grid, block, 131072, st, p, panels, row_bytes);
+  else if (steps_in_flight >= 2)
+    hipLaunchKernelGGL(floor_panel_stream_kernel<2>, grid, block, 65536, st, p, panels, row_bytes);
+  else
+    hipLaunchKernelGGL(floor_panel_stream_kernel<1>, grid, block, 32768, st, p, panels, row_bytes);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -376,13 +376,15 @@ MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_av
   const double launch = 2.6, relayout = 2.3, tile_fixed = 2.5, second_pass = 2.5, ws_rate = 2.5e6;
   MidChoice best{kVarPipe128x256w8, 1, 1e30};
   const double out_bytes = static_cast<double>(M) * N * sizeof(float);
+  // fewer rows than the 128 of a tile: the clamped rows repeat lines that are already on their way
+  const double short_rows = M >= 128 ? 1.0 : 0.6 + 0.4 * static_cast<double>(M) / 128.0;
   for (const Cand& c : cands) {
     for (int want : {1, 2, 3, 4, 6, 8}) {
       if (want > 1 && (kblocks / want < 4 || out_bytes * want > static_cast<double>(ws_avail))) continue;
       const int per = static_cast<int>(ceil_div(kblocks, want));
       const int sk = static_cast<int>(ceil_div(kblocks, per));
       const int64_t units = ceil_div(M, c.bm) * ceil_div(N, c.bn) * sk;
-      double us = launch + relayout + static_cast<double>(ceil_div(units, cus)) * (tile_fixed + per * c.step_us);
+      double us = launch + relayout + static_cast<double>(ceil_div(units, cus)) * (tile_fixed + per * c.step_us * short_rows);
       if (sk > 1) us += second_pass + (2.0 * sk + 0.5) * out_bytes / ws_rate;  // partial sums written, read back, result written
       if (us < best.us) best = MidChoice{c.variant, sk, us};
     }
@@ -409,14 +411,23 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
       // re-read the whole activation matrix from L2; K split over workgroups in two passes is twice as fast there
       // (measured at M = 128: 2112 x 7168 44 -> 22 us, 4096 x 7168 45 -> 23 us; 7168 x 2048 stays: 16 vs 19 us)
       if (M > 64 && kblocks >= 32 && ceil_div(N, 128) * 2 <= cus) v = kVarTile128x128;
-      if (M > 64 && whole_blocks) {
-        // 65 .. 128 rows: the streaming kernel's cost is its workgroups each reading all activation rows from the L2
-        // (about 6.5 TB/s over the chip); a K-split tile kernel wins when the weight matrix is narrow and K long
-        const int bn = pick_skinny_bn(N, 128, cus);
-        const double stream_us = 2.6 + static_cast<double>(ceil_div(N, bn)) * M * K / 6.5e6;
+      if (M > 32 && whole_blocks) {
+        // 33 .. 128 rows: the streaming kernel costs what is larger of its workgroups each reading all activation rows
+        // from the L2 (about 6.5 TB/s over the chip) and of its waves' K blocks, fetched one after the other: a round
+        // of 8 blocks lasts 0.15 us + 21 ns per activation row + 54 ns per weight row of the workgroup (measured at
+        // 40 .. 128 rows, 4 .. 28 weight rows, K = 2048 .. 16384).  A K-split tile kernel wins when the weight matrix
+        // is narrow and K long (2112 x 7168: 18.3 -> 15.8 us at 64 rows, 29 -> 18 us at 128; at 40 rows the streaming
+        // kernel stays ahead, 13.8 against 15.1 us)
+        const int rows = M <= 64 ? 64 : 128;
+        const int bn = pick_skinny_bn(N, rows, cus);
+        const int64_t wgs = ceil_div(N, bn);
+        const double round_us = 0.15 + 0.02125 * M + 0.054 * bn;
+        const double chain_us = round_us * static_cast<double>(ceil_div(kblocks, 8)) * static_cast<double>(ceil_div(wgs, cus));
+        const double l2_us = static_cast<double>(wgs) * M * K / 6.5e6;
+        const double stream_us = 2.6 + (l2_us > chain_us ? l2_us : chain_us);
         const MidChoice mid = pick_mid_plan(M, N, kblocks, cus, ws_avail);
         if (mid.us < stream_us) v = mid.variant, mid_splitk = mid.splitk;
-        else v = kVarSkinny128;
+        else v = M <= 64 ? kVarSkinny64 : kVarSkinny128;
       }
     } else if (whole_blocks && mode == kDense) {
       const int64_t t256 = ceil_div(M, 256) * ceil_div(N, 256);

@@ -28,6 +28,10 @@ def test_documented_choices():
     assert _lib.plan(DENSE, 128, 7168, 2048)[0] == 'skinny128'          # wide N, short K: streaming wins
     v, s, _ = _lib.plan(DENSE, 128, 2112, 7168)                          # narrow N, long K: K split over workgroups
     assert v in RING and s > 1
+    v, s, _ = _lib.plan(DENSE, 64, 2112, 7168)                           # the same from 64 rows up ...
+    assert v in RING and s > 1
+    assert _lib.plan(DENSE, 40, 2112, 7168)[0] == 'skinny64'             # ... below, streaming stays ahead
+    assert _lib.plan(DENSE, 64, 7168, 2048)[0] == 'skinny64'
     v, s, _ = _lib.plan(DENSE, 256, 7168, 16384)
     assert v in RING and s > 1
     assert _lib.plan(DENSE, 256, 7168, 2048) == ('pipe128x64', 1, 0)
