@@ -513,7 +513,7 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
                  size_t ws_bytes, int cus) {
   Resolved r{};
   const int64_t kblocks = ceil_div(K, kScaleBlock);
-  const int64_t groups = mode == kDense ? 1 : G;
+  const int64_t groups = mode == kMasked ? G : 1;  // a_s is per expert only in the masked layout; contiguous rows are one matrix
   const bool dma_ok = K < (1ll << 24) && as_sm < (1ll << 21);
   const bool usable_ws = have_ws && ws_bytes > DLB_WS_COUNTER_BYTES;
   r.pl = make_plan(mode, rows, N, K, cus, usable_ws ? ws_bytes : 0, dma_ok);
