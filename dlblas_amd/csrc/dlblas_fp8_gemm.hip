@@ -370,10 +370,14 @@ struct MidChoice {
   double us;
 };
 
+constexpr int64_t kRelayoutMinRows = 128;  // dense / grouped launches with more rows re-lay row-major activation scales first
+
 MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_avail) {
   struct Cand { int variant, bm, bn; double step_us; };
   static const Cand cands[] = {{kVarPipe128x256w8, 128, 256, 0.85}, {kVarPipe128x128, 128, 128, 0.65}, {kVarPipe128x64, 128, 64, 0.50}};
-  const double launch = 2.6, relayout = 2.3, tile_fixed = 2.5, second_pass = 2.5, ws_rate = 2.5e6;
+  const double launch = 2.6, relayout = M > kRelayoutMinRows ? 2.3 : 0.5, tile_fixed = 2.5, second_pass = 2.5, ws_rate = 3.5e6;
+  // scales fetched in place (no re-layout pass): one more line request per row and K step
+  const double scattered = M > kRelayoutMinRows ? 1.0 : 1.0 + 0.25 * static_cast<double>(M) / 128.0;
   MidChoice best{kVarPipe128x256w8, 1, 1e30};
   const double out_bytes = static_cast<double>(M) * N * sizeof(float);
   // fewer rows than the 128 of a tile: the clamped rows repeat lines that are already on their way
@@ -384,7 +388,7 @@ MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_av
       const int per = static_cast<int>(ceil_div(kblocks, want));
       const int sk = static_cast<int>(ceil_div(kblocks, per));
       const int64_t units = ceil_div(M, c.bm) * ceil_div(N, c.bn) * sk;
-      double us = launch + relayout + static_cast<double>(ceil_div(units, cus)) * (tile_fixed + per * c.step_us * short_rows);
+      double us = launch + relayout + static_cast<double>(ceil_div(units, cus)) * (tile_fixed + per * c.step_us * short_rows * scattered);
       if (sk > 1) us += second_pass + (2.0 * sk + 0.5) * out_bytes / ws_rate;  // partial sums written, read back, result written
       if (us < best.us) best = MidChoice{c.variant, sk, us};
     }
@@ -414,14 +418,15 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
       if (M > 32 && whole_blocks) {
         // 33 .. 128 rows: the streaming kernel costs what is larger of its workgroups each reading all activation rows
         // from the L2 (about 6.5 TB/s over the chip) and of its waves' K blocks, fetched one after the other: a round
-        // of 8 blocks lasts 0.15 us + 21 ns per activation row + 54 ns per weight row of the workgroup (measured at
-        // 40 .. 128 rows, 4 .. 28 weight rows, K = 2048 .. 16384).  A K-split tile kernel wins when the weight matrix
-        // is narrow and K long (2112 x 7168: 18.3 -> 15.8 us at 64 rows, 29 -> 18 us at 128; at 40 rows the streaming
-        // kernel stays ahead, 13.8 against 15.1 us)
+        // of 8 blocks lasts 0.14 us + 24 ns per activation row + 40 ns per weight row of the workgroup (measured at
+        // 33 .. 128 rows, 4 .. 28 weight rows, K = 2048 .. 16384).  A K-split tile kernel wins when the weight matrix
+        // is narrow and K long (2112 x 7168: 18.3 -> 14.1 us at 64 rows, 29 -> 17.4 us at 128; at 33 rows the streaming
+        // kernel stays ahead, 11.9 against 13.2 us)
         const int rows = M <= 64 ? 64 : 128;
         const int bn = pick_skinny_bn(N, rows, cus);
         const int64_t wgs = ceil_div(N, bn);
-        const double round_us = 0.15 + 0.02125 * M + 0.054 * bn;
+        const double m_eff = M <= 64 ? static_cast<double>(M) : 0.5 * (M + 128.0);  // the 128-row kernel computes all 8 row fragments
+        const double round_us = 0.14 + 0.0239 * m_eff + 0.04 * bn;
         const double chain_us = round_us * static_cast<double>(ceil_div(kblocks, 8)) * static_cast<double>(ceil_div(wgs, cus));
         const double l2_us = static_cast<double>(wgs) * M * K / 6.5e6;
         const double stream_us = 2.6 + (l2_us > chain_us ? l2_us : chain_us);
@@ -527,9 +532,10 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
     const size_t bytes = (static_cast<size_t>(2 + 2 * nblk) * sizeof(int32_t) + 255) / 256 * 256;
     if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
   }
-  if (is_pipelined(pl.variant) && as_sk == 1 && as_sm > 1 && usable_ws && kblocks > 1) {
+  if (is_pipelined(pl.variant) && as_sk == 1 && as_sm > 1 && usable_ws && kblocks > 1 && rows > kRelayoutMinRows) {
     // row-major activation scales: re-lay them rows-contiguous in the workspace first (a few microseconds) so the
-    // GEMM fetches 8 cache lines of scales per K step and tile instead of 256
+    // GEMM fetches 8 cache lines of scales per K step and tile instead of 256.  Up to 128 rows the extra launch costs
+    // more than the scattered scale lines (64 x 2112 x 7168: 15.9 -> 14.1 us without it)
     const int64_t rows_pad = (rows + 3) / 4 * 4;
     const int64_t need = groups * kblocks * rows_pad * static_cast<int64_t>(sizeof(float));
     if (static_cast<size_t>(need) + r.ws_used + DLB_WS_COUNTER_BYTES <= ws_bytes && rows_pad * kblocks < (1ll << 31)) {

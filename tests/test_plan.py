@@ -30,7 +30,7 @@ def test_documented_choices():
     assert v in RING and s > 1
     v, s, _ = _lib.plan(DENSE, 64, 2112, 7168)                           # the same from 64 rows up ...
     assert v in RING and s > 1
-    assert _lib.plan(DENSE, 40, 2112, 7168)[0] == 'skinny64'             # ... below, streaming stays ahead
+    assert _lib.plan(DENSE, 33, 7168, 2048)[0] == 'skinny64'             # ... a wide weight matrix streams
     assert _lib.plan(DENSE, 64, 7168, 2048)[0] == 'skinny64'
     v, s, _ = _lib.plan(DENSE, 256, 7168, 16384)
     assert v in RING and s > 1
