@@ -524,6 +524,35 @@ def permutation_workloads(dev):
     return res
 
 
+def fused_moe_workload(dev):
+    """The whole expert-contiguous MLP of one GPU's 32 local experts (dlblas_amd.kernels.fused_moe_v3.fused_moe_v3):
+    ep_scatter -> gate/up GEMM -> silu * up + quantisation -> down GEMM -> ep_gather, every intermediate allocated per call
+    as in the reference driver.  8192 tokens x top-8 over 256 experts (about one local slot per token), hidden 7168,
+    intermediate 2048.  The row also gives the sum of the five steps measured one by one, so the driver's own cost shows."""
+    import torch
+
+    from dlblas_amd.kernels.fused_moe_v3 import fused_moe_v3
+    T, H, I, E, topk = 8192, 7168, 2048, 32, 8
+    gd = torch.Generator(device=dev).manual_seed(20)
+    x_q, x_s = quantise_act(torch.randn(T, H, device=dev, generator=gd).to(torch.bfloat16))
+    ids = torch.randint(0, 256, (T, topk), device=dev, generator=gd)
+    ids[ids >= E] = -1
+    wts = torch.rand(T, topk, device=dev, generator=gd)
+    routed = torch.bincount(ids[ids >= 0], minlength=E)
+    counts = [int(c) for c in ((routed + 127) // 128 * 128).tolist()]
+    w13_q, w13_s = expert_weights(E, 2 * I, H, dev, 31)
+    w2_q, w2_s = expert_weights(E, H, I, dev, 32)
+    call = lambda: fused_moe_v3((x_q, x_s), ids, wts, (w13_q, w13_s), (w2_q, w2_s), counts)
+    call()
+    torch.cuda.synchronize()
+    ms = time_call(call, 30, 60)
+    rows, n_routed = sum(counts), int(routed.sum())
+    flops = 2.0 * n_routed * (2 * I * H + H * I)
+    return [{'workload': f'fused_moe_v3_T{T}_top{topk}_E{E}_H{H}_I{I}', 'routed_rows': n_routed, 'rows_padded': rows,
+             'us_per_call': ms * 1e3, 'TFLOPs_on_routed_rows': flops / ms / 1e9,
+             'note': 'five kernels + per-call allocation of every intermediate, timed as one call of the Python driver'}]
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 --pmc runs kept under profiles/ (None when
     no counter run for this workload has been recorded)."""
@@ -595,7 +624,7 @@ def main():
         return
 
     if args.moe_only:
-        rows = quantiser_workload(dev) + activation_workloads(dev) + permutation_workloads(dev)
+        rows = quantiser_workload(dev) + activation_workloads(dev) + permutation_workloads(dev) + fused_moe_workload(dev)
         if args.copy_calibration:
             copy_calibration(dev)
         print(json.dumps({'moe_workloads': rows}), flush=True)
@@ -679,6 +708,7 @@ def main():
         others += quantiser_workload(dev)
         others += activation_workloads(dev)
         others += permutation_workloads(dev)
+        others += fused_moe_workload(dev)
         result['other_workloads'] = others
 
     if args.copy_calibration:
