@@ -313,6 +313,11 @@ def ceilings(dev):
             lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, cus, depth, None, 0, stream)
         ms = time_call(run, 20, 20)
         res['panel_stream_GBps'][f'{depth} K steps (x 32 KB) in flight per workgroup'] = panels * 256 * row_bytes / ms / 1e6
+    for depth in (1, 4):
+        def run(depth=depth):
+            lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, 8, depth, None, 0, stream)
+        ms = time_call(run, 5, 3)
+        res['panel_stream_GBps'][f'8 workgroups only (one per XCD), {depth} K steps in flight: per workgroup'] = panels * 256 * row_bytes / ms / 1e6 / 8
     for depth in (1, 2):
         def run(depth=depth):
             lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, cus, depth, ctypes.c_void_p(hot.data_ptr()), 16, stream)
