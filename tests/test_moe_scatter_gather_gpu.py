@@ -233,3 +233,45 @@ def test_fused_moe_v3_end_to_end(dev):
     # the two early exits of the reference driver (fused_moe_v3.py:255-259)
     assert torch.equal(fused_moe_v3((x_q.to(dev), x_s.to(dev)), ids.to(dev), wts.to(dev), None, None, None).cpu(),
                        x_q.to(torch.bfloat16))
+
+
+def test_fused_moe_v3_full_size_sampled_tokens(dev):
+    """The expert MLP at one GPU's real share (8192 tokens x top-8 over 256 experts of which 32 are local, hidden 7168,
+    intermediate 2048): sampled tokens are recomputed slot by slot through the oracles (dense GEMM -> silu * up +
+    quantisation -> dense GEMM -> weighted sum) and compared under the bar of the small end-to-end test."""
+    from dlblas_amd.kernels.fused_moe_v3 import fused_moe_v3
+    print('case fused_moe_v3 full size', flush=True)
+    T, H, I, E, topk = 8192, 7168, 2048, 32, 8
+    gd = torch.Generator(device=dev).manual_seed(20)
+    x_q, x_s = helpers.quantise_act_device(torch.randn(T, H, device=dev, generator=gd).to(torch.bfloat16))
+    ids = torch.randint(0, 256, (T, topk), device=dev, generator=gd)
+    ids[ids >= E] = -1
+    wts = torch.rand(T, topk, device=dev, generator=gd)
+    routed = torch.bincount(ids[ids >= 0], minlength=E)
+    counts = [int(c) for c in ((routed + 127) // 128 * 128).tolist()]
+    w13_q, w13_s = helpers.expert_weights_device(E, 2 * I, H, dev, 31)
+    w2_q, w2_s = helpers.expert_weights_device(E, H, I, dev, 32)
+    out = fused_moe_v3((x_q, x_s), ids, wts, (w13_q, w13_s), (w2_q, w2_s), counts)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (T, H)
+    ids_c, wts_c = ids.cpu(), wts.cpu()
+    picked = [t for t in torch.randperm(T, generator=torch.Generator().manual_seed(5)).tolist() if int((ids_c[t] >= 0).sum()) > 0][:12]
+    picked.append(next(t for t in range(T) if int((ids_c[t] >= 0).sum()) == 0))   # a token no local expert takes: zeros
+    rms = float(out.float().pow(2).mean().sqrt())
+    for t in picked:
+        acc = torch.zeros(H, dtype=torch.float32)
+        for j in range(topk):
+            e = int(ids_c[t, j])
+            if e < 0:
+                continue
+            gate_up = orc.dequant_ref(x_q[t:t + 1].cpu(), x_s[t:t + 1].cpu(), w13_q[e].cpu(), w13_s[e].cpu()).to(torch.bfloat16)
+            d_q, d_s = act.silu_and_mul_post_quant_ref(gate_up)
+            down = orc.dequant_ref(d_q, d_s, w2_q[e].cpu(), w2_s[e].cpu()).to(torch.bfloat16)
+            acc = (down[0].double() * float(wts_c[t, j]) + acc.double()).float()
+        ref = acc.to(torch.bfloat16).float()
+        got = out[t].cpu().float()
+        if int((ids_c[t] >= 0).sum()) == 0:
+            assert torch.all(got == 0), f'token {t} has no local slot'
+            continue
+        assert orc.similarity_gap(got[None], ref[None]) <= 1e-4, f'token {t}'
+        assert float((got - ref).abs().max()) <= 0.05 * rms, f'token {t}'
