@@ -98,13 +98,14 @@ def fused_moe_v3(
     inter2 = w13_weight_fp8[0].size(1)  # gate and up halves side by side
     dev = tokens_q.device
 
-    def buf(shape, dtype, zero=False):
-        return (torch.zeros if zero else torch.empty)(shape, device=dev, dtype=dtype)
+    def buf(shape, dtype):
+        return torch.empty(shape, device=dev, dtype=dtype)
 
-    # Expert-sorted activations.  The spans are padded to 128 rows per expert and the GEMMs compute the padding like
-    # any other row, so it starts as zeros: stale bytes of the allocator must not reach the quantiser as NaN.
-    sorted_q = buf((rows_total, hidden), torch.uint8, zero=True).view(tokens_q.dtype)
-    sorted_scale = buf((rows_total, hidden // 128), torch.float32, zero=True)
+    # Expert-sorted activations.  The spans are padded to 128 rows per expert; the padding rows keep whatever the
+    # allocator hands out, as in the reference driver (:269-278).  The GEMMs and the quantiser treat every row on its
+    # own, so what those rows turn into (NaN included) stays in rows that ep_gather never reads.
+    sorted_q = buf((rows_total, hidden), torch.uint8).view(tokens_q.dtype)
+    sorted_scale = buf((rows_total, hidden // 128), torch.float32)
     row_expert = buf((rows_total, ), torch.int32)
     slot_row = torch.empty_like(topk_idx)
     per_expert = torch.tensor(num_recv_tokens_per_expert, dtype=torch.int32, pin_memory=True).to(dev, non_blocking=True)
