@@ -398,6 +398,15 @@ def grouped_workloads(dev):
     rows.append({'workload': f'grouped_contiguous_E{G}_T{c["tokens"]}_N{N}_K{K}', 'M_sum_padded': M_sum,
                  'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9, 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS,
                  'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS})
+    # the same GEMM as the gate/up projection of the expert MLP (N = 2 x 2048), with silu * up and the 1 x 128 quantiser
+    # in its epilogue; bytes: the bf16 output is replaced by the e4m3 activations and their scales
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_contiguous_silu_quant
+    ms = time_call(lambda: fp8_gemm_grouped_contiguous_silu_quant(a_q, a_s, w_q, w_s, m_indices), 40, 80)
+    nbytes_act = nbytes - 2 * M_sum * N + M_sum * (N // 2) + 4 * M_sum * (N // 256)
+    rows.append({'workload': f'grouped_contiguous_silu_quant_E{G}_T{c["tokens"]}_I{N // 2}_K{K}', 'M_sum_padded': M_sum,
+                 'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9, 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS,
+                 'GBps': nbytes_act / ms / 1e6, 'frac_of_hbm_peak': nbytes_act / ms / 1e6 / PEAK_HBM_GBS,
+                 'note': 'includes the allocation of its two outputs'})
     del a_q, a_s, w_q, w_s, out
     # masked (decode): valid rows uniform in [0, M_max]
     c = GROUPED_MASKED

@@ -583,6 +583,11 @@ struct Problem {
   void* ws;
   size_t ws_bytes;
   hipStream_t stream;
+  // fused gate/up epilogue (dlb_fp8_gemm_grouped_contiguous_silu_quant): c is then the e4m3 output [rows][N / 2]
+  float* act_s = nullptr;
+  int64_t act_s_sm = 0, act_s_sk = 0;
+  float act_eps = 0.f;
+  bool act = false;
 };
 
 
@@ -645,6 +650,18 @@ int run(const Problem& pr) {
   // everything that can refuse the launch is checked before the first pre-pass kernel is enqueued
   if (rs.grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)rs.grid);
   if (pl.variant == kVarExact && pr.mode != kDense) return fail(DLB_ERR_BAD_SHAPE, "exact path is dense only");
+  if (pr.act) {
+    // the fused epilogue exists for the tile-list kernel only: whole 128-blocks of K and of the output, a workspace
+    // for the list, no forced variant; anything else is the caller's cue to run the GEMM and the activation apart
+    if (pr.mode != kContiguous || !rs.tile_list || pr.K % kScaleBlock != 0 || pr.N % (2 * kScaleBlock) != 0 ||
+        pr.N * pr.K >= (1ll << 32))
+      return fail(DLB_ERR_BAD_SHAPE,
+                  "fused activation needs K %% 128 == 0, N %% 256 == 0, N K < 2^32 and a workspace for the tile list (N=%lld K=%lld)",
+                  (long long)pr.N, (long long)pr.K);
+    if (!pr.act_s || misaligned(pr.act_s, 4) || misaligned(pr.c, 8))
+      return fail(DLB_ERR_ALIGNMENT, "out_s is NULL or misaligned, or out_q is not 8-byte aligned");
+    if (pr.act_s_sm < 0 || pr.act_s_sk < 0) return fail(DLB_ERR_BAD_STRIDE, "negative out_s stride");
+  }
   if (pl.variant == kVarExact && ceil_div(pr.N, 64) > (1ll << 31) - 1) return fail(DLB_ERR_BAD_SHAPE, "N too large for the exact path");
 
   Args ar;
@@ -675,6 +692,12 @@ int run(const Problem& pr) {
   ar.kb_per_split = rs.kb_per_split;
   ar.group_m = g_knob[kKnobGroupM] > 0 ? g_knob[kKnobGroupM] : 8;
   ar.out_f32 = pr.out_dtype == DLB_OUT_F32;
+  ar.act_s = pr.act_s;
+  ar.act_s_sm = pr.act_s_sm;
+  ar.act_s_sk = pr.act_s_sk;
+  ar.act_eps = pr.act_eps;
+  ar.act_cols = static_cast<int>(pr.N / 2);
+  ar.act_q_stride = pr.N / 2;
   const size_t esz = ar.out_f32 ? 4 : 2;
   ar.vec_store = (pr.N % 4 == 0) && !misaligned(pr.c, 4 * esz);
   ar.c_vec16 = !ar.out_f32 && pr.N % 8 == 0 && !misaligned(pr.c, 16) && g_knob[kKnobEpilogue] != 2;
@@ -757,7 +780,17 @@ int run(const Problem& pr) {
         }
       } else if (pl.variant == kVarPipe256x256)
         e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
-      else if (pl.variant == kVarPipe128x256w8 && tile_list) {
+      else if (pl.variant == kVarPipe128x256w8 && tile_list && pr.act) {
+        static std::atomic<unsigned long long> lds_done{0};
+        auto kernel = fp8_gemm_contig_list_act_kernel<Pipe256x256, Pipe128x256w8>;
+        constexpr int lds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES ? Pipe256x256::LDS_BYTES : Pipe128x256w8::LDS_BYTES;
+        e = ensure_lds(kernel, lds, dev, &lds_done);
+        if (e == hipSuccess) {
+          ar.tiles_n = static_cast<int>(pr.N / 256);  // 128 output columns = 128 gate + 128 up weight rows per tile
+          hipLaunchKernelGGL(kernel, dim3(cus), dim3(Pipe256x256::NT), lds, pr.stream, ar);
+          e = hipGetLastError();
+        }
+      } else if (pl.variant == kVarPipe128x256w8 && tile_list) {
         static std::atomic<unsigned long long> lds_done{0};
         auto kernel = fp8_gemm_contig_list_kernel<Pipe256x256, Pipe128x256w8>;
         constexpr int lds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES ? Pipe256x256::LDS_BYTES : Pipe128x256w8::LDS_BYTES;
@@ -871,6 +904,22 @@ int dlb_fp8_gemm_grouped_contiguous(const void* a, const void* b, const float* a
                                     size_t workspace_bytes, void* stream) {
   dlb::Problem pr{dlb::kContiguous, a, b, a_s, b_s, c, m_indices, M_sum, N, K, G, 0, as_stride_m, as_stride_k,
                   out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  return dlb::run(pr);
+}
+
+int dlb_fp8_gemm_grouped_contiguous_silu_quant(const void* a, const void* b, const float* a_s, const float* b_s, void* out_q,
+                                               float* out_s, const int32_t* m_indices, int64_t M_sum, int64_t N, int64_t K,
+                                               int32_t G, int64_t as_stride_m, int64_t as_stride_k, int64_t os_stride_m,
+                                               int64_t os_stride_k, float eps, void* workspace, size_t workspace_bytes,
+                                               void* stream) {
+  dlb::Problem pr{dlb::kContiguous, a, b, a_s, b_s, out_q, m_indices, M_sum, N, K, G, 0, as_stride_m, as_stride_k,
+                  DLB_OUT_BF16, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  pr.act = true;
+  pr.act_s = out_s;
+  pr.act_s_sm = os_stride_m;
+  pr.act_s_sk = os_stride_k;
+  pr.act_eps = eps;
+  if (M_sum > 0 && N > 0 && G > 0 && !out_s) return dlb::fail(DLB_ERR_NULL_POINTER, "out_s is NULL");
   return dlb::run(pr);
 }
 

@@ -20,7 +20,9 @@ typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
 
 constexpr int kScaleBlock = 128;  // K (and N) extent covered by one scale; also bytes per LDS tile row
 
-enum Mode : int { kDense = 0, kContiguous = 1, kMasked = 2, kContigList = 3 };  // kContigList: contiguous, tiles from a device-built list
+// kContigList: contiguous, tiles from a device-built list.  kContigListAct: the same for the gate/up projection of an
+// expert MLP with silu(gate) * up and the 1 x 128 quantiser applied in the epilogue (see fp8_gemm_contig_list_act_kernel).
+enum Mode : int { kDense = 0, kContiguous = 1, kMasked = 2, kContigList = 3, kContigListAct = 4 };
 
 // Everything a kernel needs; passed by value as the single kernel argument.
 struct Args {
@@ -60,7 +62,24 @@ struct Args {
   int tiles_n_b;
   const int32_t* tlist;  // kContigList: [0] = 256-row tiles, [1] = 128-row tiles, then the two lists of 128-row block indices
   int tlist_cap;         //   entries per list
+  // kContigListAct: c is the e4m3 output [M][act_cols] with row stride act_q_stride (bytes); N = 2 act_cols weight rows
+  float* act_s;          //   scales of the output, element (m, j) at [m * act_s_sm + j * act_s_sk]
+  int64_t act_s_sm, act_s_sk;
+  int64_t act_q_stride;
+  int act_cols;
+  float act_eps;
 };
+
+// Arithmetic shared by the activation kernels, the quantisers and the GEMM epilogue that fuses both, so that the
+// fused and the separate paths give the same bits.
+//   act_silu_f32       gate / (1 + exp(-gate)) with the hardware exponential and reciprocal
+//   act_div_by_scale   v / s from r = 1 / s (correctly rounded, once per group): q0 = v r, then one correction with
+//                      the exact remainder, q = fma(fma(-q0, s, v), r, q0)
+__device__ __forceinline__ float act_silu_f32(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }
+__device__ __forceinline__ float act_div_by_scale(float v, float s, float r) {
+  const float q0 = v * r;
+  return fmaf(fmaf(-q0, s, v), r, q0);
+}
 
 // D = A_op * B_op^T with A_op [16 x 128] and B_op [16 x 128] e4m3; lane l supplies row (l & 15) of each
 // operand, 32 consecutive K bytes starting at 32 * (l >> 4).  Lane l receives D[4 * (l >> 4) + r][l & 15]

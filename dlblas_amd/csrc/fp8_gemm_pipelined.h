@@ -139,6 +139,11 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
   // otherwise one per 32-column fragment.
   constexpr bool kUniformW = Cfg::UNIFORM_W;
   constexpr int NS = kUniformW ? 1 : NF;
+  constexpr bool kList = MODE == kContigList || MODE == kContigListAct;
+  // Fused activation: a tile's 256 weight rows are 128 gate rows and the 128 up rows of the same output columns, so
+  // that the epilogue has silu(gate) * up of 128 columns - one quantisation group - for every row of the tile.
+  constexpr bool kAct = MODE == kContigListAct;
+  static_assert(!kAct || (BN == 256 && kUniformW), "the fused activation pairs 128 gate columns with 128 up columns");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -178,7 +183,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       mt = local % mtiles;
       nt = local / mtiles;
       m_end = min(max(p.gidx[g], 0), p.M);
-    } else if (MODE == kContigList) {
+    } else if (kList) {
       // tiles of this height come from the list the pre-pass built: entry = first 128-row block of the tile.  The
       // column tiles of one row block are adjacent in the order, so they share the activation tile in L2.
       const int cnt = p.tlist[BM == 256 ? 0 : 1];
@@ -212,8 +217,10 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       }
     }
     g = __builtin_amdgcn_readfirstlane(g);
-    const int m0 = __builtin_amdgcn_readfirstlane(MODE == kContigList ? m_first : mt * BM);
-    const int n0 = __builtin_amdgcn_readfirstlane(n_base + nt * BN);
+    const int m0 = __builtin_amdgcn_readfirstlane(kList ? m_first : mt * BM);
+    // fused activation: n0 is the first OUTPUT column of the tile; weight row of tile column c: see w_row below
+    const int n0 = __builtin_amdgcn_readfirstlane(kAct ? nt * (BN / 2) : n_base + nt * BN);
+    auto w_row = [&](int c) { return c < BN / 2 ? n0 + c : p.act_cols + n0 + c - BN / 2; };
 
     const int64_t esz = p.out_f32 ? 4 : 2;
     const bool sliced = MODE == kDense && p.splitk > 1;
@@ -226,13 +233,14 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       as_tile += static_cast<int64_t>(g) * p.as_gs;
       c_base += static_cast<int64_t>(g) * p.c_gs * esz;
     }
-    const uint8_t* b_tile =
-        p.b + static_cast<int64_t>(g) * p.b_gs + static_cast<int64_t>(n0) * p.K + static_cast<int64_t>(kb_first) * kScaleBlock;
+    const uint8_t* b_tile = p.b + static_cast<int64_t>(g) * p.b_gs + static_cast<int64_t>(kAct ? 0 : n0) * p.K +
+                            static_cast<int64_t>(kb_first) * kScaleBlock;
     // weight scales: lane i of the wave fetches the scale of the wave's fragment (i & 3) (fragment 0 beyond NF)
     const float* bs_g = p.b_s + static_cast<int64_t>(g) * p.bs_gs + kb_first;
     const int bs_frag = (lane & 3) < NF ? (lane & 3) : 0;
     const uint32_t bs_off =
-        static_cast<uint32_t>(min((n0 + wn0 + 32 * bs_frag) / kScaleBlock, p.nblocks - 1)) * static_cast<uint32_t>(p.kblocks) * 4u;
+        static_cast<uint32_t>(min((kAct ? w_row(wn0 + 32 * bs_frag) : n0 + wn0 + 32 * bs_frag) / kScaleBlock, p.nblocks - 1)) *
+        static_cast<uint32_t>(p.kblocks) * 4u;
 
     // DMA addressing.  Instruction j of this wave fills LDS rows 8 (j WAVES + wave) .. + 7; lane i fills physical
     // chunk (i & 7) of row (i >> 3), which holds logical chunk (i & 7) ^ swizzle(row).  WAVES is even, so the
@@ -255,7 +263,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       a_off[j] = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, a_last)) * uK + dma_chunk;
 #pragma unroll
     for (int j = 0; j < Cfg::B_INST; ++j)
-      b_off[j] = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, b_last)) * uK + dma_chunk;
+      b_off[j] = static_cast<uint32_t>(kAct ? w_row(dma_row + 8 * j * WAVES) : min(dma_row + 8 * j * WAVES, b_last)) * uK + dma_chunk;
 #pragma unroll
     for (int j = 0; j < Cfg::S_INST; ++j)
       s_off[j] = static_cast<uint32_t>(min((j * WAVES + wave) * 64 + lane, a_last)) * static_cast<uint32_t>(p.as_sm) * 4u;
@@ -569,6 +577,70 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     }
 
     // epilogue: lane holds c[m0 + wm0 + 32 mi + (lane & 31)][n0 + wn0 + 32 ni + 8 u + 4 (lane >> 5) + 0..3], u = 0..3
+    if constexpr (kAct) {
+      // The tile goes to LDS as the bf16 matrix the unfused GEMM would have written ([BM][gate 128 | up 128], 8-byte
+      // chunks XOR-ed with an even function of the row so that the 32 rows of a store instruction spread over the
+      // banks and 16-byte reads stay whole), then 16 lanes per row compute silu(gate) * up rounded to bf16 and quantise
+      // the 128 values exactly as silu_and_mul + per_token_group_quant_fp8 do (moe_activation.h, fp8_quant.h).
+      constexpr int kRowB = BN * 2;
+      static_assert(BM * kRowB <= Cfg::LDS_BYTES, "the staged tile fits in the ring");
+      __syncthreads();  // every wave is done reading the ring
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) {
+        const int row = wm0 + mi * 32 + l32;
+        const int x = (row & 31) << 1;
+#pragma unroll
+        for (int ni = 0; ni < NF; ++ni)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const v4f v = {acc[mi][ni][4 * u], acc[mi][ni][4 * u + 1], acc[mi][ni][4 * u + 2], acc[mi][ni][4 * u + 3]};
+            const int chunk = (wn0 + ni * 32 + u * 8 + h * 4) >> 2;
+            *reinterpret_cast<v4bf*>(smem + row * kRowB + ((chunk ^ x) << 3)) = __builtin_convertvector(v, v4bf);
+          }
+      }
+      __syncthreads();
+      const int sub = tid & 15;
+      uint8_t* q_out = static_cast<uint8_t*>(p.c);
+#pragma unroll 2
+      for (int r0 = 0; r0 < BM; r0 += Cfg::NT / 16) {
+        const int row = r0 + (tid >> 4);
+        const int x = (row & 31) << 1;
+        const v4i graw = *reinterpret_cast<const v4i*>(smem + row * kRowB + (((2 * sub) ^ x) << 3));
+        const v4i uraw = *reinterpret_cast<const v4i*>(smem + row * kRowB + (((BN / 4 / 2 + 2 * sub) ^ x) << 3));
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t gw = static_cast<uint32_t>(graw[i]), uw = static_cast<uint32_t>(uraw[i]);
+          const float g0 = __builtin_bit_cast(float, gw << 16), g1 = __builtin_bit_cast(float, gw & 0xffff0000u);
+          const float u0 = __builtin_bit_cast(float, uw << 16), u1 = __builtin_bit_cast(float, uw & 0xffff0000u);
+          v[2 * i] = static_cast<float>(static_cast<__bf16>(act_silu_f32(g0) * u0));
+          v[2 * i + 1] = static_cast<float>(static_cast<__bf16>(act_silu_f32(g1) * u1));
+        }
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+#pragma unroll
+        for (int off = 8; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 16));
+        const float scale = fmaxf(amax, p.act_eps) / 448.0f;
+        const float inv_scale = 1.0f / scale;
+        int packed[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          float c4[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) c4[j] = fminf(fmaxf(act_div_by_scale(v[4 * i + j], scale, inv_scale), -448.0f), 448.0f);
+          int wd = __builtin_amdgcn_cvt_pk_fp8_f32(c4[0], c4[1], 0, false);
+          wd = __builtin_amdgcn_cvt_pk_fp8_f32(c4[2], c4[3], wd, true);
+          packed[i] = wd;
+        }
+        const int m = m0 + row;
+        if (row < BM && m < m_end) {
+          *reinterpret_cast<v2i*>(q_out + static_cast<int64_t>(m) * p.act_q_stride + n0 + sub * 8) = v2i{packed[0], packed[1]};
+          if (sub == 0) p.act_s[static_cast<int64_t>(m) * p.act_s_sm + static_cast<int64_t>(n0 / kScaleBlock) * p.act_s_sk] = scale;
+        }
+      }
+      continue;
+    }
     if (sliced) {
       // first pass of split-K: the slice's sums go to the workspace as an fp32 [M][N] matrix of their own;
       // fp8_splitk_reduce_kernel, launched behind this kernel on the same stream, adds the slices in index order
@@ -710,6 +782,19 @@ __global__ void __launch_bounds__(CfgA::NT) fp8_gemm_contig_list_kernel(const Ar
   const int total_a = p.tlist[0] * p.tiles_n;
   const int first_b = (static_cast<int>(blockIdx.x) + gridDim.x - total_a % gridDim.x) % gridDim.x;
   pipelined_body<CfgB, kContigList>(p, smem, first_b, 0, p.tiles_n, 0);
+}
+
+// The gate/up projection of an expert MLP with the activation and the quantiser of its output fused into the epilogue
+// (dlblas/kernels/fused_moe_v3.py:307-334 as one kernel): weights [G][2 I][K] with the gate rows first, output
+// e4m3 [M][I] + scales [M][I / 128].  Same tile lists and schedule as fp8_gemm_contig_list_kernel; tiles_n = I / 128.
+template <class CfgA, class CfgB>
+__global__ void __launch_bounds__(CfgA::NT) fp8_gemm_contig_list_act_kernel(const Args p) {
+  static_assert(CfgA::NT == CfgB::NT && CfgA::BN == CfgB::BN, "both tile heights use the same workgroup shape and width");
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  pipelined_body<CfgA, kContigListAct>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
+  const int total_a = p.tlist[0] * p.tiles_n;
+  const int first_b = (static_cast<int>(blockIdx.x) + gridDim.x - total_a % gridDim.x) % gridDim.x;
+  pipelined_body<CfgB, kContigListAct>(p, smem, first_b, 0, p.tiles_n, 0);
 }
 
 template <class CfgA, class CfgB>

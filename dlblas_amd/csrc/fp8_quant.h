@@ -75,10 +75,7 @@ __device__ __forceinline__ void quant_load8(const void* x, int64_t elem, float (
 // rounding is within 2^-47 of v / s, so q is the correctly rounded quotient unless v / s lies that close to a
 // midpoint between two floats; 3 instructions instead of the 10 of a full division, which made the quantisers
 // ALU-bound.
-__device__ __forceinline__ float div_by_scale(float v, float s, float r) {
-  const float q0 = v * r;
-  return fmaf(fmaf(-q0, s, v), r, q0);
-}
+__device__ __forceinline__ float div_by_scale(float v, float s, float r) { return act_div_by_scale(v, s, r); }
 
 template <int IN>
 __global__ void __launch_bounds__(256) fp8_quant_1x128_kernel(const QuantArgs p) {

@@ -39,7 +39,7 @@ __device__ __forceinline__ float round_to_input(float v) {
 // do (fast exp and approximate division of the Triton build).  The result is rounded to a 8- or 11-bit significand
 // right after, so the choice shows in about one result in 10^4; the correctly rounded forms cost 3x the instructions
 // and made this HBM-bound kernel ALU-bound.
-__device__ __forceinline__ float silu_f32(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }
+__device__ __forceinline__ float silu_f32(float g) { return act_silu_f32(g); }
 
 template <int IN>
 __device__ __forceinline__ void act_store8(void* out, int64_t elem, const float (&v)[8]) {

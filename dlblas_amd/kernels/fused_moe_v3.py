@@ -2,7 +2,8 @@
 package: ``ep_scatter`` (:95-158), ``ep_gather`` (:199-233) and the driver ``fused_moe_v3`` (:246-343) with the same
 positional signatures.  Differences a caller can observe: destination rows are handed out in token-major order instead
 of atomic order (both satisfy the contract that ``output_index`` names the row each slot was copied to), and the
-driver fuses silu_and_mul with the quantiser and skips the scale re-layout the reference needs for its GEMM.
+driver runs the gate/up GEMM, silu_and_mul and the quantiser as one kernel (same bits as the three steps) and skips
+the scale re-layout the reference needs for its GEMM.
 """
 from typing import List, Optional, Tuple
 
@@ -10,7 +11,7 @@ import torch
 
 from .. import _lib
 from .activation import silu_and_mul_post_quant
-from .fp8_gemm_grouped import m_grouped_fp8_gemm_nt_contiguous
+from .fp8_gemm_grouped import fp8_gemm_grouped_contiguous_silu_quant, m_grouped_fp8_gemm_nt_contiguous
 
 
 @torch.library.custom_op('dlblas::ep_scatter', mutates_args=('expert_start_loc', 'output_tensor', 'output_tensor_scale',
@@ -112,10 +113,17 @@ def fused_moe_v3(
     first_row = torch.empty_like(per_expert)
     ep_scatter(tokens_q, tokens_scale, topk_idx, per_expert, first_row, sorted_q, sorted_scale, row_expert, slot_row)
 
-    gate_up = buf((rows_total, inter2), torch.bfloat16)
-    m_grouped_fp8_gemm_nt_contiguous((sorted_q, sorted_scale), w13_weight_fp8, gate_up, row_expert)
-    act_q, act_scale = silu_and_mul_post_quant(gate_up, 128)
-    del gate_up
+    # gate/up projection, silu(gate) * up and the 1 x 128 quantiser: one kernel where the library has it (the bf16
+    # [rows, 2 I] intermediate then never reaches memory), else the three steps of the reference (:307-334)
+    fused = fp8_gemm_grouped_contiguous_silu_quant(sorted_q, sorted_scale, w13_weight_fp8[0], w13_weight_fp8[1], row_expert,
+                                                   column_major_scales=True)  # the layout the down GEMM reads in place
+    if fused is not None:
+        act_q, act_scale = fused
+    else:
+        gate_up = buf((rows_total, inter2), torch.bfloat16)
+        m_grouped_fp8_gemm_nt_contiguous((sorted_q, sorted_scale), w13_weight_fp8, gate_up, row_expert)
+        act_q, act_scale = silu_and_mul_post_quant(gate_up, 128)
+        del gate_up
     down = buf((rows_total, hidden), torch.bfloat16)
     m_grouped_fp8_gemm_nt_contiguous((act_q, act_scale), w2_weight_fp8, down, row_expert)
 

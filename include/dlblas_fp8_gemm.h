@@ -45,7 +45,7 @@
 extern "C" {
 #endif
 
-#define DLB_ABI_VERSION 2
+#define DLB_ABI_VERSION 3
 
 /* output element type of C */
 #define DLB_OUT_BF16 0
@@ -140,6 +140,31 @@ int dlb_fp8_gemm_grouped_contiguous(const void* a, const void* b, const float* a
                                     int64_t M_sum, int64_t N, int64_t K, int32_t G,
                                     int64_t as_stride_m, int64_t as_stride_k,
                                     int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The gate/up projection of an expert MLP with its activation and the quantiser of the result fused into the GEMM:
+ * one kernel instead of the sequence grouped GEMM -> silu_and_mul -> per_token_group_quant_fp8 of
+ * dlblas/kernels/fused_moe_v3.py:307-334, with the same bits (the bf16 rounding of the GEMM output, the activation
+ * in bf16 and the 1 x 128 quantiser are reproduced in the epilogue).  The bf16 [M_sum, N] intermediate never reaches
+ * memory.
+ *
+ *   a, a_s, m_indices, G, as_stride_*   as dlb_fp8_gemm_grouped_contiguous
+ *   b      [G, N, K]                    e4m3fn; N = 2 I weight rows per expert, the I gate rows first, then the I up rows
+ *   b_s    [G, N/128, K/128]            fp32
+ *   out_q  [M_sum, I]                   e4m3fn, row stride I:  quant(silu(gate) * up)
+ *   out_s  [M_sum, I/128]               fp32, element (m, j) at [m * os_stride_m + j * os_stride_k]
+ *   eps                                 lower bound of a group's amax (the reference passes 1e-10)
+ *
+ * Needs K % 128 == 0, N % 256 == 0, N * K < 2^32 and a workspace (the tile list of the expert-contiguous path lives
+ * there); otherwise DLB_ERR_BAD_SHAPE is returned, nothing is enqueued, and the caller runs the three steps apart.
+ * Rows of blocks whose m_indices entry is negative are not written.
+ */
+int dlb_fp8_gemm_grouped_contiguous_silu_quant(const void* a, const void* b, const float* a_s, const float* b_s,
+                                               void* out_q, float* out_s, const int32_t* m_indices,
+                                               int64_t M_sum, int64_t N, int64_t K, int32_t G,
+                                               int64_t as_stride_m, int64_t as_stride_k,
+                                               int64_t os_stride_m, int64_t os_stride_k, float eps,
+                                               void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Grouped GEMM, fixed-capacity buffers with a valid-row count per expert.  Replaces
