@@ -425,6 +425,31 @@ def grouped_workloads(dev):
     rows.append({'workload': f'grouped_masked_E{G}_Mmax{M_max}_N{N}_K{K}', 'valid_rows': valid,
                  'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9, 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS,
                  'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS})
+    del w_q, w_s, out
+    # the first half of the decode MoE layer (gate/up projection: 2 x 2048 weight rows, K = 7168) with the same masked_m:
+    # masked GEMM + masked activation + quantiser as one kernel, and as the two kernels it replaces
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_masked_silu_quant
+    from dlblas_amd.kernels.moe import silu_and_mul_masked_post_quant_fwd
+    N, K = GROUPED_CONTIGUOUS['N'], GROUPED_CONTIGUOUS['K']
+    a_q, a_s = quantise_act(torch.randn(G * M_max, K, device=dev, generator=gd).to(torch.bfloat16))
+    a_q, a_s = a_q.reshape(G, M_max, K), a_s.reshape(G, M_max, K // 128)
+    w_q, w_s = expert_weights(G, N, K, dev, 25)
+    q = torch.empty(G, M_max, N // 2, dtype=torch.float8_e4m3fn, device=dev)
+    q_s = torch.empty(G, M_max, N // 256, dtype=torch.float32, device=dev)
+    gate_up = torch.empty(G, M_max, N, dtype=torch.bfloat16, device=dev)
+
+    def two_steps():
+        fp8_gemm_grouped_masked(a_q, a_s, w_q, w_s, gate_up, mm, hint)
+        silu_and_mul_masked_post_quant_fwd(gate_up, q, q_s, 128, mm)
+
+    ms2 = time_call(two_steps, 60, 150)
+    ms = time_call(lambda: fp8_gemm_grouped_masked_silu_quant(a_q, a_s, w_q, w_s, q, q_s, mm, hint), 60, 150)
+    flops = 2.0 * valid * N * K
+    nbytes = valid * K + G * N * K + 4 * valid * (K // 128) + 4 * G * (N // 128) * (K // 128) + valid * (N // 2) + 4 * valid * (N // 256) + 4 * G
+    rows.append({'workload': f'grouped_masked_silu_quant_E{G}_Mmax{M_max}_I{N // 2}_K{K}', 'valid_rows': valid,
+                 'us_per_launch': ms * 1e3, 'us_as_two_kernels': ms2 * 1e3, 'TFLOPs': flops / ms / 1e9,
+                 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS, 'GBps': nbytes / ms / 1e6,
+                 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS})
     return rows
 
 

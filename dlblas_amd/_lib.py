@@ -12,7 +12,7 @@ import torch
 
 from ._build import LIB_PATH
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 OUT_BF16, OUT_F32 = 0, 1
 WS_COUNTER_BYTES = 65536
 WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
@@ -34,6 +34,8 @@ SYMBOLS = {
     (ctypes.c_int, [_c_vp] * 6 + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 2 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_grouped_contiguous_silu_quant':
     (ctypes.c_int, [_c_vp] * 7 + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 4 + [ctypes.c_float, _c_vp, _c_sz, _c_vp]),
+    'dlb_fp8_gemm_grouped_masked_silu_quant':
+    (ctypes.c_int, [_c_vp] * 7 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 6 + [ctypes.c_float, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_grouped_masked':
     (ctypes.c_int, [_c_vp] * 6 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 3 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_quant_1x128': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
@@ -263,6 +265,23 @@ def gemm_masked(a, b, a_s, b_s, c, masked_m, expected_m, M_max, N, K, G, as_sg, 
             lib.dlb_fp8_gemm_grouped_masked(_ptr(a), _ptr(b), _ptr(a_s), _ptr(b_s), _ptr(c), _ptr(masked_m),
                                             int(expected_m), M_max, N, K, G, as_sg, as_sm, as_sk,
                                             out_code(c.dtype), _ptr(ws), ws.numel(), ctypes.c_void_p(stream)))
+
+
+def gemm_masked_silu_quant(a, b, a_s, b_s, out_q, out_s, masked_m, expected_m, M_max, N, K, G, as_sg, as_sm, as_sk, eps) -> bool:
+    """The fused masked gate/up GEMM + up * silu(gate) + 1 x 128 quantiser.  False when the library has no fused kernel
+    for the shape (ERR_BAD_SHAPE): nothing was enqueued and the caller runs the steps apart."""
+    _require_gpu(a, b, a_s, b_s, out_q, out_s, masked_m)
+    lib = load()
+    with torch.cuda.device(a.device):
+        stream, ws = _stream_and_ws(a)
+        rc = lib.dlb_fp8_gemm_grouped_masked_silu_quant(_ptr(a), _ptr(b), _ptr(a_s), _ptr(b_s), _ptr(out_q), _ptr(out_s),
+                                                        _ptr(masked_m), int(expected_m), M_max, N, K, G, as_sg, as_sm, as_sk,
+                                                        out_s.stride(0), out_s.stride(1), out_s.stride(2), float(eps),
+                                                        _ptr(ws), ws.numel(), ctypes.c_void_p(stream))
+        if rc == ERR_BAD_SHAPE:
+            return False
+        check(rc)
+        return True
 
 
 IN_CODES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}

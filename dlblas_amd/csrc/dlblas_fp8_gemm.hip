@@ -583,9 +583,10 @@ struct Problem {
   void* ws;
   size_t ws_bytes;
   hipStream_t stream;
-  // fused gate/up epilogue (dlb_fp8_gemm_grouped_contiguous_silu_quant): c is then the e4m3 output [rows][N / 2]
+  // fused gate/up epilogue (dlb_fp8_gemm_grouped_{contiguous,masked}_silu_quant): c is then the e4m3 output
+  // [rows][N / 2] ([G][rows][N / 2] masked)
   float* act_s = nullptr;
-  int64_t act_s_sm = 0, act_s_sk = 0;
+  int64_t act_s_sg = 0, act_s_sm = 0, act_s_sk = 0;
   float act_eps = 0.f;
   bool act = false;
 };
@@ -651,16 +652,17 @@ int run(const Problem& pr) {
   if (rs.grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)rs.grid);
   if (pl.variant == kVarExact && pr.mode != kDense) return fail(DLB_ERR_BAD_SHAPE, "exact path is dense only");
   if (pr.act) {
-    // the fused epilogue exists for the tile-list kernel only: whole 128-blocks of K and of the output, a workspace
-    // for the list, no forced variant; anything else is the caller's cue to run the GEMM and the activation apart
-    if (pr.mode != kContiguous || !rs.tile_list || pr.K % kScaleBlock != 0 || pr.N % (2 * kScaleBlock) != 0 ||
-        pr.N * pr.K >= (1ll << 32))
+    // the fused epilogue exists for the tile-list kernel (contiguous) and the 128 x 256 ring kernel (masked) only:
+    // whole 128-blocks of K and of the output, a workspace for the list, no forced variant; anything else is the
+    // caller's cue to run the GEMM and the activation apart
+    const bool kernel_ok = pr.mode == kContiguous ? rs.tile_list : pr.mode == kMasked && pl.variant == kVarPipe128x256w8;
+    if (!kernel_ok || pr.K % kScaleBlock != 0 || pr.N % (2 * kScaleBlock) != 0 || pr.N * pr.K >= (1ll << 32))
       return fail(DLB_ERR_BAD_SHAPE,
-                  "fused activation needs K %% 128 == 0, N %% 256 == 0, N K < 2^32 and a workspace for the tile list (N=%lld K=%lld)",
-                  (long long)pr.N, (long long)pr.K);
+                  "fused activation needs K %% 128 == 0, N %% 256 == 0, N K < 2^32%s (N=%lld K=%lld)",
+                  pr.mode == kContiguous ? " and a workspace for the tile list" : "", (long long)pr.N, (long long)pr.K);
     if (!pr.act_s || misaligned(pr.act_s, 4) || misaligned(pr.c, 8))
       return fail(DLB_ERR_ALIGNMENT, "out_s is NULL or misaligned, or out_q is not 8-byte aligned");
-    if (pr.act_s_sm < 0 || pr.act_s_sk < 0) return fail(DLB_ERR_BAD_STRIDE, "negative out_s stride");
+    if (pr.act_s_sm < 0 || pr.act_s_sk < 0 || pr.act_s_sg < 0) return fail(DLB_ERR_BAD_STRIDE, "negative out_s stride");
   }
   if (pl.variant == kVarExact && ceil_div(pr.N, 64) > (1ll << 31) - 1) return fail(DLB_ERR_BAD_SHAPE, "N too large for the exact path");
 
@@ -693,6 +695,7 @@ int run(const Problem& pr) {
   ar.group_m = g_knob[kKnobGroupM] > 0 ? g_knob[kKnobGroupM] : 8;
   ar.out_f32 = pr.out_dtype == DLB_OUT_F32;
   ar.act_s = pr.act_s;
+  ar.act_s_gs = pr.act_s_sg;
   ar.act_s_sm = pr.act_s_sm;
   ar.act_s_sk = pr.act_s_sk;
   ar.act_eps = pr.act_eps;
@@ -800,7 +803,9 @@ int run(const Problem& pr) {
           hipLaunchKernelGGL(kernel, dim3(cus), dim3(Pipe256x256::NT), lds, pr.stream, ar);  // one resident workgroup per CU
           e = hipGetLastError();
         }
-      } else if (pl.variant == kVarPipe128x256w8)
+      } else if (pl.variant == kVarPipe128x256w8 && pr.act)
+        e = launch_pipelined<Pipe128x256w8, kMaskedAct>(ar, g, dev, pr.stream);  // N / 256 column tiles, as the plain GEMM
+      else if (pl.variant == kVarPipe128x256w8)
         e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g_dense, dev, pr.stream);
       else if (pl.variant == kVarPipe128x128)
         e = launch_pipelined_mode<Pipe128x128>(pr.mode, ar, g, dev, pr.stream);
@@ -920,6 +925,24 @@ int dlb_fp8_gemm_grouped_contiguous_silu_quant(const void* a, const void* b, con
   pr.act_s_sk = os_stride_k;
   pr.act_eps = eps;
   if (M_sum > 0 && N > 0 && G > 0 && !out_s) return dlb::fail(DLB_ERR_NULL_POINTER, "out_s is NULL");
+  return dlb::run(pr);
+}
+
+int dlb_fp8_gemm_grouped_masked_silu_quant(const void* a, const void* b, const float* a_s, const float* b_s, void* out_q,
+                                           float* out_s, const int32_t* masked_m, int32_t expected_m, int64_t M_max,
+                                           int64_t N, int64_t K, int32_t G, int64_t as_stride_g, int64_t as_stride_m,
+                                           int64_t as_stride_k, int64_t os_stride_g, int64_t os_stride_m, int64_t os_stride_k,
+                                           float eps, void* workspace, size_t workspace_bytes, void* stream) {
+  (void)expected_m;
+  dlb::Problem pr{dlb::kMasked, a, b, a_s, b_s, out_q, masked_m, M_max, N, K, G, as_stride_g, as_stride_m, as_stride_k,
+                  DLB_OUT_BF16, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  pr.act = true;
+  pr.act_s = out_s;
+  pr.act_s_sg = os_stride_g;
+  pr.act_s_sm = os_stride_m;
+  pr.act_s_sk = os_stride_k;
+  pr.act_eps = eps;
+  if (M_max > 0 && N > 0 && G > 0 && !out_s) return dlb::fail(DLB_ERR_NULL_POINTER, "out_s is NULL");
   return dlb::run(pr);
 }
 

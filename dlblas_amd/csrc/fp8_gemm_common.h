@@ -22,7 +22,8 @@ constexpr int kScaleBlock = 128;  // K (and N) extent covered by one scale; also
 
 // kContigList: contiguous, tiles from a device-built list.  kContigListAct: the same for the gate/up projection of an
 // expert MLP with silu(gate) * up and the 1 x 128 quantiser applied in the epilogue (see fp8_gemm_contig_list_act_kernel).
-enum Mode : int { kDense = 0, kContiguous = 1, kMasked = 2, kContigList = 3, kContigListAct = 4 };
+// kMaskedAct: that epilogue on the masked layout, with the masked activation's two roundings (dlblas/kernels/moe.py:256-257).
+enum Mode : int { kDense = 0, kContiguous = 1, kMasked = 2, kContigList = 3, kContigListAct = 4, kMaskedAct = 5 };
 
 // Everything a kernel needs; passed by value as the single kernel argument.
 struct Args {
@@ -62,9 +63,10 @@ struct Args {
   int tiles_n_b;
   const int32_t* tlist;  // kContigList: [0] = 256-row tiles, [1] = 128-row tiles, then the two lists of 128-row block indices
   int tlist_cap;         //   entries per list
-  // kContigListAct: c is the e4m3 output [M][act_cols] with row stride act_q_stride (bytes); N = 2 act_cols weight rows
-  float* act_s;          //   scales of the output, element (m, j) at [m * act_s_sm + j * act_s_sk]
-  int64_t act_s_sm, act_s_sk;
+  // kContigListAct / kMaskedAct: c is the e4m3 output [G][M][act_cols] with row stride act_q_stride (bytes);
+  // N = 2 act_cols weight rows
+  float* act_s;          //   scales of the output, element (g, m, j) at [g * act_s_gs + m * act_s_sm + j * act_s_sk]
+  int64_t act_s_gs, act_s_sm, act_s_sk;
   int64_t act_q_stride;
   int act_cols;
   float act_eps;

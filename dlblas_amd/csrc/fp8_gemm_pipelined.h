@@ -142,7 +142,8 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
   constexpr bool kList = MODE == kContigList || MODE == kContigListAct;
   // Fused activation: a tile's 256 weight rows are 128 gate rows and the 128 up rows of the same output columns, so
   // that the epilogue has silu(gate) * up of 128 columns - one quantisation group - for every row of the tile.
-  constexpr bool kAct = MODE == kContigListAct;
+  constexpr bool kAct = MODE == kContigListAct || MODE == kMaskedAct;
+  constexpr bool kMaskedLike = MODE == kMasked || MODE == kMaskedAct;
   static_assert(!kAct || (BN == 256 && kUniformW), "the fused activation pairs 128 gate columns with 128 up columns");
 
   const int tid = threadIdx.x;
@@ -160,7 +161,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
 
   for (int vb = vb_first;; vb += gridDim.x) {
     int g = 0, mt = 0, nt, m_end, m_first = -1, split = 0;
-    if (MODE == kMasked) {
+    if (kMaskedLike) {
       // The tile count is only known on the device, so the grid is persistent; the hardware deals consecutive
       // workgroups to the 8 XCDs in turn.  Of every 32 consecutive tiles each XCD takes 4 consecutive ones: the row
       // tiles of an expert, which are adjacent in the order and read the same weight tile, meet in one L2, and the
@@ -228,7 +229,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     const uint8_t* a_tile = p.a + static_cast<int64_t>(m0) * p.K + static_cast<int64_t>(kb_first) * kScaleBlock;
     const float* as_tile = p.a_s + static_cast<int64_t>(m0) * p.as_sm + static_cast<int64_t>(kb_first) * p.as_sk;
     char* c_base = static_cast<char*>(p.c);
-    if (MODE == kMasked) {
+    if (kMaskedLike) {
       a_tile += static_cast<int64_t>(g) * p.a_gs;
       as_tile += static_cast<int64_t>(g) * p.as_gs;
       c_base += static_cast<int64_t>(g) * p.c_gs * esz;
@@ -601,6 +602,11 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       __syncthreads();
       const int sub = tid & 15;
       uint8_t* q_out = static_cast<uint8_t*>(p.c);
+      float* s_out = p.act_s;
+      if (kMaskedLike) {
+        q_out += static_cast<int64_t>(g) * p.M * p.act_q_stride;
+        s_out += static_cast<int64_t>(g) * p.act_s_gs;
+      }
 #pragma unroll 2
       for (int r0 = 0; r0 < BM; r0 += Cfg::NT / 16) {
         const int row = r0 + (tid >> 4);
@@ -613,8 +619,13 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
           const uint32_t gw = static_cast<uint32_t>(graw[i]), uw = static_cast<uint32_t>(uraw[i]);
           const float g0 = __builtin_bit_cast(float, gw << 16), g1 = __builtin_bit_cast(float, gw & 0xffff0000u);
           const float u0 = __builtin_bit_cast(float, uw << 16), u1 = __builtin_bit_cast(float, uw & 0xffff0000u);
-          v[2 * i] = static_cast<float>(static_cast<__bf16>(act_silu_f32(g0) * u0));
-          v[2 * i + 1] = static_cast<float>(static_cast<__bf16>(act_silu_f32(g1) * u1));
+          if (kMaskedLike) {  // the masked activation rounds silu(gate) before the product (moe.py:256-257)
+            v[2 * i] = static_cast<float>(static_cast<__bf16>(u0 * static_cast<float>(static_cast<__bf16>(act_silu_f32(g0)))));
+            v[2 * i + 1] = static_cast<float>(static_cast<__bf16>(u1 * static_cast<float>(static_cast<__bf16>(act_silu_f32(g1)))));
+          } else {
+            v[2 * i] = static_cast<float>(static_cast<__bf16>(act_silu_f32(g0) * u0));
+            v[2 * i + 1] = static_cast<float>(static_cast<__bf16>(act_silu_f32(g1) * u1));
+          }
         }
         float amax = 0.f;
 #pragma unroll
@@ -636,7 +647,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         const int m = m0 + row;
         if (row < BM && m < m_end) {
           *reinterpret_cast<v2i*>(q_out + static_cast<int64_t>(m) * p.act_q_stride + n0 + sub * 8) = v2i{packed[0], packed[1]};
-          if (sub == 0) p.act_s[static_cast<int64_t>(m) * p.act_s_sm + static_cast<int64_t>(n0 / kScaleBlock) * p.act_s_sk] = scale;
+          if (sub == 0) s_out[static_cast<int64_t>(m) * p.act_s_sm + static_cast<int64_t>(n0 / kScaleBlock) * p.act_s_sk] = scale;
         }
       }
       continue;

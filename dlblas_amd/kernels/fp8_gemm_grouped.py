@@ -137,6 +137,50 @@ def fp8_gemm_grouped_masked(a, a_s, w, w_s, out, masked_m, expected_m=0):
     grouped_masked_op(a, a_s, w, w_s, out, masked_m, int(expected_m))
 
 
+@torch.library.custom_op('dlblas::fp8_gemm_grouped_masked_silu_quant', mutates_args=('out_q', 'out_s'), device_types='cuda')
+def grouped_masked_silu_quant_op(a: torch.Tensor, a_s: torch.Tensor, w: torch.Tensor, w_s: torch.Tensor, out_q: torch.Tensor,
+                                 out_s: torch.Tensor, masked_m: torch.Tensor, expected_m: int, eps: float) -> bool:
+    G, N, K = w.shape
+    return _lib.gemm_masked_silu_quant(a, w, a_s, w_s, out_q, out_s, masked_m, expected_m, a.size(1), N, K, G, a_s.stride(0),
+                                       a_s.stride(1), a_s.stride(2), eps)
+
+
+@grouped_masked_silu_quant_op.register_fake
+def _(a, a_s, w, w_s, out_q, out_s, masked_m, expected_m, eps):
+    return True
+
+
+def fp8_gemm_grouped_masked_silu_quant(a, a_s, w13, w13_s, out_q, out_s, masked_m, expected_m=0, eps: float = 1e-10) -> bool:
+    """The first half of the masked (low-latency) expert MLP in one kernel: ``m_grouped_fp8_gemm_nt_masked`` into a
+    bf16 buffer followed by ``silu_and_mul_masked_post_quant_fwd`` (dlblas/layers/moe/ep_moe.py:199-251), with the same
+    bits and without the bf16 [G, M_max, 2 I] intermediate in memory.  ``w13`` is [G, 2 I, K] with the gate rows first;
+    ``out_q`` e4m3fn [G, M_max, I] and ``out_s`` float32 [G, M_max, I / 128] (any strides) are written for the first
+    ``masked_m[g]`` rows of every expert and keep their content elsewhere.  Returns False, with nothing written, when
+    the library has no fused kernel for the shape: the caller then runs the two steps apart."""
+    for name, t, dt in (('a', a, torch.float8_e4m3fn), ('w13', w13, torch.float8_e4m3fn), ('a_s', a_s, torch.float32),
+                        ('w13_s', w13_s, torch.float32), ('out_q', out_q, torch.float8_e4m3fn), ('out_s', out_s, torch.float32)):
+        if t.dtype != dt:
+            raise TypeError(f'{name} must be {dt}, got {t.dtype}')
+    assert a.is_contiguous() and w13.is_contiguous() and out_q.is_contiguous(), 'Input tensors must be contiguous'
+    assert w13_s.is_contiguous(), 'Scaling factor tensors must be contiguous'
+    if w13.dim() != 3 or a.dim() != 3 or a.size(0) != w13.size(0) or a.size(2) != w13.size(2):
+        raise ValueError(f'a must be [G, M_max, K] and w13 [G, 2 I, K], got {tuple(a.shape)} and {tuple(w13.shape)}')
+    G, N, K = w13.shape
+    M_max = a.size(1)
+    if N % (2 * BLOCK) != 0 or K % BLOCK != 0:
+        return False
+    inter = N // 2
+    if tuple(w13_s.shape) != (G, N // BLOCK, K // BLOCK) or tuple(a_s.shape) != (G, M_max, K // BLOCK):
+        raise ValueError('a_s must be [G, M_max, K / 128] and w13_s [G, 2 I / 128, K / 128]')
+    if tuple(out_q.shape) != (G, M_max, inter) or tuple(out_s.shape) != (G, M_max, inter // BLOCK):
+        raise ValueError(f'out_q must be [{G}, {M_max}, {inter}] and out_s [{G}, {M_max}, {inter // BLOCK}]')
+    if masked_m.dtype != torch.int32 or tuple(masked_m.shape) != (G, ) or not masked_m.is_contiguous():
+        raise ValueError('masked_m must be a contiguous int32 vector with one entry per expert')
+    if G == 0 or M_max == 0:
+        return True
+    return grouped_masked_silu_quant_op(a, a_s, w13, w13_s, out_q, out_s, masked_m, int(expected_m), float(eps))
+
+
 # --- deep_gemm-compatible positional entry points (what the reference's shims call) --------------------------
 
 

@@ -66,17 +66,25 @@ def low_latency_experts(
     128 x 128 block scales; masked_m [G] int32.  Returns down_output [G, M_max, K] in out_dtype; rows at or beyond
     masked_m[g] are not written (they hold whatever the allocation held, as in the reference).
     """
-    from .fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
+    from .fp8_gemm_grouped import fp8_gemm_grouped_masked_silu_quant, m_grouped_fp8_gemm_nt_masked
     a, a_s = hidden_states_fp8
     num_groups, m, k = a.shape
     n = gate_up_weight.size(1)
     expected_m = min(expected_m, m)
-    gateup_output = torch.empty((num_groups, m, n), device=a.device, dtype=out_dtype)
-    m_grouped_fp8_gemm_nt_masked((a, a_s), (gate_up_weight, gate_up_scale), gateup_output, masked_m, expected_m)
     down_input = torch.empty((num_groups, m, n // 2), device=a.device, dtype=gate_down_weight.dtype)
-    down_input_scale = torch.empty((num_groups, m, n // 2 // block_size), device=a.device, dtype=torch.float32)
-    silu_and_mul_masked_post_quant_fwd(gateup_output, down_input, down_input_scale, block_size, masked_m)
-    del gateup_output
+    fused = False
+    if out_dtype == torch.bfloat16 and block_size == 128 and n % 256 == 0 and masked_m.dtype == torch.int32:
+        # one kernel for GEMM + activation + quantiser, same bits; its scales go out with the rows of a K block
+        # contiguous, the layout the second GEMM reads without a re-layout pass
+        down_input_scale = torch.empty((num_groups, n // 2 // block_size, m), device=a.device, dtype=torch.float32).transpose(1, 2)
+        fused = fp8_gemm_grouped_masked_silu_quant(a, a_s, gate_up_weight, gate_up_scale, down_input, down_input_scale,
+                                                   masked_m, expected_m)
+    if not fused:
+        gateup_output = torch.empty((num_groups, m, n), device=a.device, dtype=out_dtype)
+        m_grouped_fp8_gemm_nt_masked((a, a_s), (gate_up_weight, gate_up_scale), gateup_output, masked_m, expected_m)
+        down_input_scale = torch.empty((num_groups, m, n // 2 // block_size), device=a.device, dtype=torch.float32)
+        silu_and_mul_masked_post_quant_fwd(gateup_output, down_input, down_input_scale, block_size, masked_m)
+        del gateup_output
     down_output = torch.empty((num_groups, m, gate_down_weight.size(1)), device=a.device, dtype=out_dtype)
     m_grouped_fp8_gemm_nt_masked((down_input, down_input_scale), (gate_down_weight, gate_down_scale), down_output, masked_m,
                                  expected_m)

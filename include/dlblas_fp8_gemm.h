@@ -45,7 +45,7 @@
 extern "C" {
 #endif
 
-#define DLB_ABI_VERSION 3
+#define DLB_ABI_VERSION 4
 
 /* output element type of C */
 #define DLB_OUT_BF16 0
@@ -191,6 +191,30 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
                                 int64_t M_max, int64_t N, int64_t K, int32_t G,
                                 int64_t as_stride_g, int64_t as_stride_m, int64_t as_stride_k,
                                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The gate/up projection of the masked (low-latency) expert MLP with its activation and the quantiser of the result
+ * fused into the GEMM: one kernel instead of m_grouped_fp8_gemm_nt_masked -> silu_and_mul_masked_post_quant_fwd
+ * (dlblas/layers/moe/ep_moe.py:199-251), with the same bits (the bf16 rounding of the GEMM output, the two bf16
+ * roundings of the masked activation, dlblas/kernels/moe.py:256-257, and the 1 x 128 quantiser are reproduced in the
+ * epilogue).  The bf16 [G, M_max, N] intermediate never reaches memory.
+ *
+ *   a, a_s, masked_m, expected_m, G, as_stride_*   as dlb_fp8_gemm_grouped_masked
+ *   b      [G, N, K]                    e4m3fn; N = 2 I weight rows per expert, the I gate rows first, then the I up rows
+ *   b_s    [G, N/128, K/128]            fp32
+ *   out_q  [G, M_max, I]                e4m3fn, contiguous:  quant(up * silu(gate))
+ *   out_s  [G, M_max, I/128]            fp32, element (g, m, j) at [g * os_stride_g + m * os_stride_m + j * os_stride_k]
+ *   eps                                 lower bound of a group's amax (the reference uses 1e-10)
+ *
+ * Rows at or beyond masked_m[g] of out_q and out_s are not written.  Needs K % 128 == 0, N % 256 == 0 and
+ * N * K < 2^32; otherwise DLB_ERR_BAD_SHAPE is returned, nothing is enqueued, and the caller runs the two steps apart.
+ */
+int dlb_fp8_gemm_grouped_masked_silu_quant(const void* a, const void* b, const float* a_s, const float* b_s,
+                                           void* out_q, float* out_s, const int32_t* masked_m, int32_t expected_m,
+                                           int64_t M_max, int64_t N, int64_t K, int32_t G,
+                                           int64_t as_stride_g, int64_t as_stride_m, int64_t as_stride_k,
+                                           int64_t os_stride_g, int64_t os_stride_m, int64_t os_stride_k, float eps,
+                                           void* workspace, size_t workspace_bytes, void* stream);
 
 /* element type of the quantiser input */
 #define DLB_IN_BF16 0

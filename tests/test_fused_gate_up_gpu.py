@@ -88,3 +88,93 @@ def test_fused_full_size(dev):
     assert fused is not None
     assert torch.equal(fused[0].view(torch.uint8), ref_q.view(torch.uint8))
     assert torch.equal(fused[1], ref_s)
+
+
+# --- masked (low-latency) layout: m_grouped_fp8_gemm_nt_masked -> silu_and_mul_masked_post_quant_fwd in one kernel ----
+
+
+def _masked_both(dev, a_q, a_s, w_q, w_s, masked_m, col_major_out=False):
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_masked_silu_quant, m_grouped_fp8_gemm_nt_masked
+    from dlblas_amd.kernels.moe import silu_and_mul_masked_post_quant_fwd
+    G, M_max, _ = a_q.shape
+    inter = w_q.size(1) // 2
+    sentinel_q, sentinel_s = 0x5a, -7.0
+    q = torch.full((G, M_max, inter), sentinel_q, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    if col_major_out:
+        s = torch.full((G, inter // 128, M_max), sentinel_s, device=dev).transpose(1, 2)
+    else:
+        s = torch.full((G, M_max, inter // 128), sentinel_s, device=dev)
+    ok = fp8_gemm_grouped_masked_silu_quant(a_q, a_s, w_q, w_s, q, s, masked_m, expected_m=int(masked_m.max()))
+    gate_up = torch.zeros(G, M_max, 2 * inter, dtype=torch.bfloat16, device=dev)
+    m_grouped_fp8_gemm_nt_masked((a_q, a_s), (w_q, w_s), gate_up, masked_m, int(masked_m.max()))
+    ref_q = torch.full((G, M_max, inter), sentinel_q, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    ref_s = torch.full((G, M_max, inter // 128), sentinel_s, device=dev)
+    silu_and_mul_masked_post_quant_fwd(gate_up, ref_q, ref_s, 128, masked_m)
+    torch.cuda.synchronize()
+    return ok, (q, s), (ref_q, ref_s)
+
+
+@pytest.mark.parametrize('masked,M_max,inter,K,col_major_out', [
+    ([5], 128, 128, 128, False),
+    ([0, 128, 77], 128, 256, 512, False),
+    ([200, 1, 256, 129], 256, 384, 1024, True),
+    ([300, 0, 45], 384, 128, 2048, False),
+    ([64, 64, 64, 64, 64, 64, 64, 64, 3], 64, 512, 256, True),
+])
+def test_masked_fused_equals_the_two_steps(dev, masked, M_max, inter, K, col_major_out):
+    print(f'case fused masked gate/up masked_m={masked} M_max={M_max} I={inter} K={K}', flush=True)
+    G = len(masked)
+    g = helpers.gen(700 + M_max + inter + K)
+    qs = [orc.quant_act_1x128((torch.randn(M_max, K, generator=g) * 1.5).to(torch.bfloat16)) for _ in range(G)]
+    a_q, a_s = torch.stack([x[0] for x in qs]).to(dev), torch.stack([x[1] for x in qs]).to(dev)
+    ws = [orc.quant_weight_128x128((torch.randn(2 * inter, K, generator=g) * 0.05).to(torch.bfloat16)) for _ in range(G)]
+    w_q, w_s = torch.stack([w[0] for w in ws]).to(dev), torch.stack([w[1] for w in ws]).to(dev)
+    masked_m = torch.tensor(masked, dtype=torch.int32, device=dev)
+    ok, (q, s), (ref_q, ref_s) = _masked_both(dev, a_q, a_s, w_q, w_s, masked_m, col_major_out)
+    assert ok
+    # every byte and every scale: valid rows equal the two-step result, rows beyond masked_m keep the sentinels
+    assert torch.equal(q.view(torch.uint8), ref_q.view(torch.uint8)), 'quantised codes differ'
+    assert torch.equal(s, ref_s), 'scales differ'
+    valid = torch.arange(M_max, device=dev)[None, :] < masked_m[:, None]
+    assert (ref_s[~valid] == -7.0).all() and (ref_s[valid] > 0).all()
+
+
+def test_masked_shapes_without_a_fused_kernel_are_declined(dev):
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_masked_silu_quant
+    a_q = torch.zeros(2, 128, 192, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)   # K % 128 != 0
+    a_s = torch.ones(2, 128, 2, device=dev)
+    w_q = torch.zeros(2, 256, 192, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    w_s = torch.ones(2, 2, 2, device=dev)
+    q = torch.zeros(2, 128, 128, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    s = torch.zeros(2, 128, 1, device=dev)
+    masked_m = torch.tensor([3, 4], dtype=torch.int32, device=dev)
+    assert fp8_gemm_grouped_masked_silu_quant(a_q, a_s, w_q, w_s, q, s, masked_m) is False
+    torch.cuda.synchronize()
+    assert (s == 0).all()
+
+
+def test_masked_fused_full_size_and_low_latency_experts(dev):
+    """The decode MoE layer's compute on one GPU at the size of the masked benchmark row (32 experts x 256 slots,
+    2 x 2048 x 7168 and 7168 x 2048): the fused first half equals the two steps bit for bit, and low_latency_experts,
+    which uses it, equals the three-kernel sequence of the reference driver."""
+    print('case fused masked gate/up full size', flush=True)
+    from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
+    from dlblas_amd.kernels.moe import low_latency_experts
+    G, M_max, inter, K = 32, 256, 2048, 7168
+    gd = torch.Generator(device=dev).manual_seed(31)
+    x = torch.randn(G * M_max, K, device=dev, generator=gd).to(torch.bfloat16)
+    a_q, a_s = helpers.quantise_act_device(x)
+    a_q, a_s = a_q.view(G, M_max, K), a_s.view(G, M_max, K // 128).contiguous()
+    w13_q, w13_s = helpers.expert_weights_device(G, 2 * inter, K, dev, 32)
+    w2_q, w2_s = helpers.expert_weights_device(G, K, inter, dev, 33)
+    masked_m = torch.randint(0, M_max + 1, (G, ), generator=torch.Generator().manual_seed(34)).to(torch.int32).to(dev)
+    ok, (q, s), (ref_q, ref_s) = _masked_both(dev, a_q, a_s, w13_q, w13_s, masked_m)
+    assert ok
+    assert torch.equal(q.view(torch.uint8), ref_q.view(torch.uint8))
+    assert torch.equal(s, ref_s)
+    out = low_latency_experts((a_q, a_s), w13_q, w13_s, w2_q, w2_s, masked_m, int(masked_m.max()))
+    ref = torch.zeros(G, M_max, K, dtype=torch.bfloat16, device=dev)
+    m_grouped_fp8_gemm_nt_masked((ref_q, ref_s), (w2_q, w2_s), ref, masked_m, int(masked_m.max()))
+    torch.cuda.synchronize()
+    valid = torch.arange(M_max, device=dev)[None, :] < masked_m[:, None]
+    assert torch.equal(out[valid], ref[valid])
