@@ -383,7 +383,7 @@ MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_av
   // fewer rows than the 128 of a tile: the clamped rows repeat lines that are already on their way
   const double short_rows = M >= 128 ? 1.0 : 0.6 + 0.4 * static_cast<double>(M) / 128.0;
   for (const Cand& c : cands) {
-    for (int want : {1, 2, 3, 4, 6, 8}) {
+    for (int want : {1, 2, 3, 4, 5, 6, 7, 8}) {
       if (want > 1 && (kblocks / want < 4 || out_bytes * want > static_cast<double>(ws_avail))) continue;
       const int per = static_cast<int>(ceil_div(kblocks, want));
       const int sk = static_cast<int>(ceil_div(kblocks, per));
