@@ -589,7 +589,7 @@ def fused_moe_workload(dev):
     flops = 2.0 * n_routed * (2 * I * H + H * I)
     return [{'workload': f'fused_moe_v3_T{T}_top{topk}_E{E}_H{H}_I{I}', 'routed_rows': n_routed, 'rows_padded': rows,
              'us_per_call': ms * 1e3, 'TFLOPs_on_routed_rows': flops / ms / 1e9,
-             'note': 'five kernels + per-call allocation of every intermediate, timed as one call of the Python driver'}]
+             'note': 'scatter, fused gate/up GEMM, down GEMM, gather with their pre-passes + per-call allocation of every intermediate, timed as one call of the Python driver'}]
 
 
 def measured_traffic(workload):
