@@ -587,9 +587,27 @@ def fused_moe_workload(dev):
     ms = time_call(call, 30, 60)
     rows, n_routed = sum(counts), int(routed.sum())
     flops = 2.0 * n_routed * (2 * I * H + H * I)
-    return [{'workload': f'fused_moe_v3_T{T}_top{topk}_E{E}_H{H}_I{I}', 'routed_rows': n_routed, 'rows_padded': rows,
-             'us_per_call': ms * 1e3, 'TFLOPs_on_routed_rows': flops / ms / 1e9,
-             'note': 'scatter, fused gate/up GEMM, down GEMM, gather with their pre-passes + per-call allocation of every intermediate, timed as one call of the Python driver'}]
+    out = [{'workload': f'fused_moe_v3_T{T}_top{topk}_E{E}_H{H}_I{I}', 'routed_rows': n_routed, 'rows_padded': rows,
+            'us_per_call': ms * 1e3, 'TFLOPs_on_routed_rows': flops / ms / 1e9,
+            'note': 'scatter, fused gate/up GEMM, down GEMM, gather with their pre-passes + per-call allocation of every intermediate, timed as one call of the Python driver'}]
+    # the decode counterpart: the masked expert MLP (dlblas_amd.kernels.moe.low_latency_experts) on 32 experts x 256
+    # row slots with masked_m uniform in [0, 256]: fused gate/up GEMM + activation + quantiser, then the down GEMM
+    from dlblas_amd.kernels.moe import low_latency_experts
+    M_max = GROUPED_MASKED['M_max']
+    masked_m = torch.randint(0, M_max + 1, (E, ), generator=torch.Generator().manual_seed(20), dtype=torch.int32)
+    a_q, a_s = quantise_act(torch.randn(E * M_max, H, device=dev, generator=gd).to(torch.bfloat16))
+    a_q, a_s = a_q.reshape(E, M_max, H), a_s.reshape(E, M_max, H // 128)
+    mm, hint = masked_m.to(dev), int(masked_m.float().mean())
+    call = lambda: low_latency_experts((a_q, a_s), w13_q, w13_s, w2_q, w2_s, mm, hint)
+    call()
+    torch.cuda.synchronize()
+    ms = time_call(call, 30, 60)
+    valid = int(masked_m.sum())
+    out.append({'workload': f'low_latency_experts_E{E}_Mmax{M_max}_H{H}_I{I}', 'valid_rows': valid, 'us_per_call': ms * 1e3,
+                'TFLOPs_on_valid_rows': 2.0 * valid * (2 * I * H + H * I) / ms / 1e9,
+                'weight_GBps': E * 3 * I * H / ms / 1e6,
+                'note': 'fused masked gate/up GEMM + down GEMM + per-call allocation of the intermediates; the weights (1.41 GB) are read once'})
+    return out
 
 
 def measured_traffic(workload):
