@@ -271,10 +271,43 @@ def decode_floor(dev, N=7168, K=2048, copies=24):
             tried[f'{per_cu} wg/cu x {depth} loads'] = time_call(reader(cus * per_cu, depth), 240, 240) * 1e3
     best = min(tried, key=tried.get)
     read_us = time_call(reader(cus * int(best.split()[0]), int(best.split()[3])), 480, 1500) * 1e3
+    del bufs
     return {'empty_launch_us': empty_ms * 1e3, 'read_only_us': read_us, 'read_only_GBps': N * K / read_us / 1e3,
-            'read_only_shape': best, 'bytes_read': N * K,
+            'read_only_shape': best, 'bytes_read': N * K, 'gemm_16_rows_graph_replay_us': decode_graph_replay(dev, 16, N, K, copies),
             'note': 'bench-only kernels (bench_kernels/floor_kernels.hip), same rotation of weight buffers and same launch '
-                    'loop as the decode rows; read_only = fastest of 9 shapes of a kernel that only loads the weight bytes'}
+                    'loop as the decode rows; read_only = fastest of 9 shapes of a kernel that only loads the weight bytes; '
+                    'graph_replay = the GEMM itself, 48 launches captured in a HIP graph and replayed'}
+
+
+def decode_graph_replay(dev, M, N, K, copies):
+    """Per-launch time of the decode GEMM when 48 launches over the rotating weight buffers are captured in a HIP graph
+    and the graph is replayed: what is left of a launch when the host's part of it is taken away."""
+    import torch
+    a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=copies)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    per_graph = 2 * copies
+    with torch.cuda.stream(side):
+        launch = DenseLauncher(a_q, a_s, ws, out)  # its calls carry the side stream
+        for _ in range(per_graph):
+            launch()
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(per_graph):
+                launch()
+        for _ in range(30):
+            graph.replay()
+        side.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(side)
+        for _ in range(10):
+            graph.replay()
+        stop.record(side)
+        side.synchronize()
+    torch.cuda.current_stream().wait_stream(side)
+    return start.elapsed_time(stop) / (10 * per_graph) * 1e3
 
 
 def ceilings(dev):
