@@ -320,7 +320,7 @@ def ceilings(dev):
     lib = ctypes.CDLL(FLOOR_LIB)
     lib.floor_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
     lib.floor_panel_stream.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
-                                       ctypes.c_void_p]
+                                       ctypes.c_int, ctypes.c_void_p]
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     g = torch.Generator().manual_seed(20)
@@ -341,22 +341,26 @@ def ceilings(dev):
     panels, row_bytes = 256, 7168
     mat = torch.randint(0, 255, (panels * 256 * row_bytes, ), dtype=torch.uint8, device=dev)
     hot = torch.randint(0, 255, (16 * 256 * row_bytes, ), dtype=torch.uint8, device=dev)
-    for depth in (1, 2, 4):
-        def run(depth=depth):
-            lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, cus, depth, None, 0, stream)
-        ms = time_call(run, 20, 20)
-        res['panel_stream_GBps'][f'{depth} K steps (x 32 KB) in flight per workgroup'] = panels * 256 * row_bytes / ms / 1e6
-    for depth in (1, 4):
-        def run(depth=depth):
-            lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, 8, depth, None, 0, stream)
-        ms = time_call(run, 5, 3)
-        res['panel_stream_GBps'][f'8 workgroups only (one per XCD), {depth} K steps in flight: per workgroup'] = panels * 256 * row_bytes / ms / 1e6 / 8
-    for depth in (1, 2):
-        def run(depth=depth):
-            lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, cus, depth, ctypes.c_void_p(hot.data_ptr()), 16, stream)
-        ms = time_call(run, 20, 20)
-        res['panel_stream_GBps'][f'{depth} K steps in flight, plus a shared (L2-resident) 256-row panel per step: HBM panel bytes only'] = \
-            panels * 256 * row_bytes / ms / 1e6
+    for hint in (0, 1):
+        tag = ', non-temporal loads' if hint else ''
+        for depth in (1, 2, 4):
+            def run(depth=depth, hint=hint):
+                lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, cus, depth, None, 0, hint, stream)
+            ms = time_call(run, 20, 20)
+            res['panel_stream_GBps'][f'{depth} K steps (x 32 KB) in flight per workgroup{tag}'] = panels * 256 * row_bytes / ms / 1e6
+        for depth in (1, 4):
+            def run(depth=depth, hint=hint):
+                lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, 8, depth, None, 0, hint, stream)
+            ms = time_call(run, 5, 3)
+            res['panel_stream_GBps'][f'8 workgroups only (one per XCD), {depth} K steps in flight{tag}: per workgroup'] = \
+                panels * 256 * row_bytes / ms / 1e6 / 8
+        for depth in (1, 2):
+            def run(depth=depth, hint=hint):
+                lib.floor_panel_stream(ctypes.c_void_p(mat.data_ptr()), panels, row_bytes, cus, depth, ctypes.c_void_p(hot.data_ptr()), 16, hint,
+                                       stream)
+            ms = time_call(run, 20, 20)
+            res['panel_stream_GBps'][f'{depth} K steps in flight, plus a shared (L2-resident) 256-row panel per step{tag}: HBM panel bytes only'] = \
+                panels * 256 * row_bytes / ms / 1e6
     res['note'] = ('mfma_loop: pairs of v_mfma_f32_32x32x64_f8f6f4 + 16 scale FMAs from registers, 8 waves per CU, no memory '
                    'traffic except the optional LDS reads (the prefill kernel issues 3 per pair); peak 5000 TFLOP/s. '
                    'panel_stream: one workgroup per CU pulls 256 x 7168-byte panels from HBM through the LDS DMA path, '

