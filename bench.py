@@ -462,12 +462,23 @@ def grouped_workloads(dev):
     rows.append({'workload': f'grouped_masked_E{G}_Mmax{M_max}_N{N}_K{K}', 'valid_rows': valid,
                  'us_per_launch': ms * 1e3, 'TFLOPs': flops / ms / 1e9, 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS,
                  'GBps': nbytes / ms / 1e6, 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS})
-    del w_q, w_s, out
-    # the first half of the decode MoE layer (gate/up projection: 2 x 2048 weight rows, K = 7168) with the same masked_m:
-    # masked GEMM + masked activation + quantiser as one kernel, and as the two kernels it replaces
-    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_masked_silu_quant
+    return rows
+
+
+def masked_gate_up_workload(dev):
+    """The first half of the decode MoE layer (gate/up projection: 2 x 2048 weight rows, K = 7168) on 32 experts x 256 row
+    slots with masked_m uniform in [0, 256]: masked GEMM + masked activation + quantiser as one kernel, and as the two
+    kernels it replaces."""
+    import torch
+
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_masked, fp8_gemm_grouped_masked_silu_quant
     from dlblas_amd.kernels.moe import silu_and_mul_masked_post_quant_fwd
+    c = GROUPED_MASKED
+    G, M_max = c['G'], c['M_max']
     N, K = GROUPED_CONTIGUOUS['N'], GROUPED_CONTIGUOUS['K']
+    masked_m = torch.randint(0, M_max + 1, (G, ), generator=torch.Generator().manual_seed(20), dtype=torch.int32)
+    mm, hint, valid = masked_m.to(dev), int(masked_m.float().mean()), int(masked_m.sum())
+    gd = torch.Generator(device=dev).manual_seed(23)
     a_q, a_s = quantise_act(torch.randn(G * M_max, K, device=dev, generator=gd).to(torch.bfloat16))
     a_q, a_s = a_q.reshape(G, M_max, K), a_s.reshape(G, M_max, K // 128)
     w_q, w_s = expert_weights(G, N, K, dev, 25)
@@ -483,11 +494,10 @@ def grouped_workloads(dev):
     ms = time_call(lambda: fp8_gemm_grouped_masked_silu_quant(a_q, a_s, w_q, w_s, q, q_s, mm, hint), 60, 150)
     flops = 2.0 * valid * N * K
     nbytes = valid * K + G * N * K + 4 * valid * (K // 128) + 4 * G * (N // 128) * (K // 128) + valid * (N // 2) + 4 * valid * (N // 256) + 4 * G
-    rows.append({'workload': f'grouped_masked_silu_quant_E{G}_Mmax{M_max}_I{N // 2}_K{K}', 'valid_rows': valid,
-                 'us_per_launch': ms * 1e3, 'us_as_two_kernels': ms2 * 1e3, 'TFLOPs': flops / ms / 1e9,
-                 'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS, 'GBps': nbytes / ms / 1e6,
-                 'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS})
-    return rows
+    return [{'workload': f'grouped_masked_silu_quant_E{G}_Mmax{M_max}_I{N // 2}_K{K}', 'valid_rows': valid,
+             'us_per_launch': ms * 1e3, 'us_as_two_kernels': ms2 * 1e3, 'TFLOPs': flops / ms / 1e9,
+             'frac_of_fp8_peak': flops / ms / 1e9 / PEAK_FP8_TFLOPS, 'GBps': nbytes / ms / 1e6,
+             'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS}]
 
 
 def quantiser_workload(dev):
@@ -718,7 +728,8 @@ def main():
         return
 
     if args.moe_only:
-        rows = quantiser_workload(dev) + activation_workloads(dev) + permutation_workloads(dev) + fused_moe_workload(dev)
+        rows = (quantiser_workload(dev) + activation_workloads(dev) + permutation_workloads(dev) + masked_gate_up_workload(dev) +
+                fused_moe_workload(dev))
         if args.copy_calibration:
             copy_calibration(dev)
         print(json.dumps({'moe_workloads': rows}), flush=True)
@@ -802,6 +813,7 @@ def main():
         others += quantiser_workload(dev)
         others += activation_workloads(dev)
         others += permutation_workloads(dev)
+        others += masked_gate_up_workload(dev)
         others += fused_moe_workload(dev)
         result['other_workloads'] = others
 
