@@ -12,7 +12,7 @@ import torch
 
 from ._build import LIB_PATH
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 OUT_BF16, OUT_F32 = 0, 1
 WS_COUNTER_BYTES = 65536
 WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
@@ -34,6 +34,8 @@ SYMBOLS = {
     (ctypes.c_int, [_c_vp] * 6 + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 2 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_grouped_contiguous_silu_quant':
     (ctypes.c_int, [_c_vp] * 7 + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 4 + [ctypes.c_float, _c_vp, _c_sz, _c_vp]),
+    'dlb_fp8_gemm_grouped_contiguous_gather_silu_quant':
+    (ctypes.c_int, [_c_vp] * 8 + [_c_i64] * 4 + [_c_i32] + [_c_i64] * 4 + [ctypes.c_float, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_grouped_masked_silu_quant':
     (ctypes.c_int, [_c_vp] * 7 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 6 + [ctypes.c_float, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_gemm_grouped_masked':
@@ -53,6 +55,9 @@ SYMBOLS = {
     (ctypes.c_int, [_c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_vp, _c_vp, ctypes.c_int, _c_vp,
                     _c_i64, _c_vp, _c_i64, _c_i64, _c_vp, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
                     _c_i64, _c_vp, _c_sz, _c_vp]),
+    'dlb_ep_scatter_rows':
+    (ctypes.c_int, [_c_vp, ctypes.c_int, _c_i64, _c_i64, _c_vp, _c_vp, ctypes.c_int, _c_vp, _c_vp, _c_i64, _c_vp, ctypes.c_int,
+                    _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp, _c_sz, _c_vp]),
     'dlb_ep_gather':
     (ctypes.c_int, [_c_vp, ctypes.c_int, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp, ctypes.c_int,
                     _c_i64, _c_i64, _c_vp, ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
@@ -256,6 +261,22 @@ def gemm_contiguous_silu_quant(a, b, a_s, b_s, out_q, out_s, m_indices, M_sum, N
         return True
 
 
+def gemm_contiguous_gather_silu_quant(a, b, a_s, b_s, out_q, out_s, m_indices, a_row_index, N, K, G, eps) -> bool:
+    """gemm_contiguous_silu_quant whose row r is row a_row_index[r] of a / a_s.  False when the library declines the shape."""
+    _require_gpu(a, b, a_s, b_s, out_q, out_s, m_indices, a_row_index)
+    lib = load()
+    with torch.cuda.device(a.device):
+        stream, ws = _stream_and_ws(a)
+        rc = lib.dlb_fp8_gemm_grouped_contiguous_gather_silu_quant(
+            _ptr(a), _ptr(b), _ptr(a_s), _ptr(b_s), _ptr(out_q), _ptr(out_s), _ptr(m_indices), _ptr(a_row_index), a.size(0),
+            m_indices.numel(), N, K, G, a_s.stride(0), a_s.stride(1), out_s.stride(0), out_s.stride(1), float(eps), _ptr(ws),
+            ws.numel(), ctypes.c_void_p(stream))
+        if rc == ERR_BAD_SHAPE:
+            return False
+        check(rc)
+        return True
+
+
 def gemm_masked(a, b, a_s, b_s, c, masked_m, expected_m, M_max, N, K, G, as_sg, as_sm, as_sk):
     _require_gpu(a, b, a_s, b_s, c, masked_m)
     lib = load()
@@ -356,6 +377,23 @@ def ep_scatter(recv_x, recv_x_scale, recv_topk, counts, expert_start_loc, out, o
     with torch.cuda.device(recv_x.device):
         check(load().dlb_ep_scatter(*ep_scatter_args(recv_x, recv_x_scale, recv_topk, counts, expert_start_loc, out, out_scale,
                                                      m_indices, output_index)))
+
+
+def ep_scatter_rows(recv_topk, counts, expert_start_loc, m_indices, src_row, output_index):
+    """dlb_ep_scatter_rows: the tables of ep_scatter and the source token of every destination row; no row is moved."""
+    lib = load()
+    _require_gpu(recv_topk, counts, expert_start_loc, m_indices, src_row, output_index)
+    T, topk = recv_topk.shape
+    E = counts.shape[0]
+    with torch.cuda.device(recv_topk.device):
+        stream, ws = _stream_and_ws(recv_topk)
+        need = lib.dlb_ep_scatter_workspace_bytes(T, topk, E)
+        if need > ws.numel():
+            raise ValueError(f'ep_scatter needs {need} bytes of workspace, the per-stream buffer holds {ws.numel()}')
+        check(lib.dlb_ep_scatter_rows(_ptr(recv_topk), _idx_code(recv_topk), recv_topk.stride(0), recv_topk.stride(1), _ptr(counts),
+                                      _ptr(expert_start_loc), _idx_code(expert_start_loc), _ptr(m_indices), _ptr(src_row),
+                                      m_indices.numel(), _ptr(output_index), _idx_code(output_index), output_index.stride(0),
+                                      output_index.stride(1), T, topk, E, _ptr(ws), ws.numel(), ctypes.c_void_p(stream)))
 
 
 def ep_gather_args(inp, topk_ids, topk_weight, index, out):

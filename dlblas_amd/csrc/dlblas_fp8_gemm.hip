@@ -515,7 +515,7 @@ struct Resolved {
 };
 
 Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as_sm, int64_t as_sk, bool have_ws,
-                 size_t ws_bytes, int cus) {
+                 size_t ws_bytes, int cus, bool gather_scales = false) {
   Resolved r{};
   const int64_t kblocks = ceil_div(K, kScaleBlock);
   const int64_t groups = mode == kMasked ? G : 1;  // a_s is per expert only in the masked layout; contiguous rows are one matrix
@@ -532,7 +532,9 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
     const size_t bytes = (static_cast<size_t>(2 + 2 * nblk) * sizeof(int32_t) + 255) / 256 * 256;
     if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
   }
-  if (is_pipelined(pl.variant) && as_sk == 1 && as_sm > 1 && usable_ws && kblocks > 1 && rows > kRelayoutMinRows) {
+  // gather_scales: the re-layout pass also brings the rows into the GEMM's order, so it runs whatever the strides
+  if (is_pipelined(pl.variant) && usable_ws &&
+      (gather_scales ? kblocks > 0 : as_sk == 1 && as_sm > 1 && kblocks > 1 && rows > kRelayoutMinRows)) {
     // row-major activation scales: re-lay them rows-contiguous in the workspace first (a few microseconds) so the
     // GEMM fetches 8 cache lines of scales per K step and tile instead of 256.  Up to 128 rows the extra launch costs
     // more than the scattered scale lines (64 x 2112 x 7168: 15.9 -> 14.1 us without it)
@@ -587,6 +589,10 @@ struct Problem {
   // [rows][N / 2] ([G][rows][N / 2] masked)
   float* act_s = nullptr;
   int64_t act_s_sg = 0, act_s_sm = 0, act_s_sk = 0;
+  // ... reading its activation rows through a table (dlb_fp8_gemm_grouped_contiguous_gather_silu_quant): row r of the
+  // GEMM is row a_rows[r] of a [a_src_rows][K]; a_s has a_src_rows rows too
+  const int32_t* a_rows = nullptr;
+  int64_t a_src_rows = 0;
   float act_eps = 0.f;
   bool act = false;
 };
@@ -646,7 +652,8 @@ int run(const Problem& pr) {
   if (cus < 0) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
 
   if (pr.ws && misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
-  const Resolved rs = resolve(pr.mode, pr.rows, pr.N, pr.K, pr.G, pr.as_sm, pr.as_sk, pr.ws != nullptr, pr.ws_bytes, cus);
+  const Resolved rs = resolve(pr.mode, pr.rows, pr.N, pr.K, pr.G, pr.as_sm, pr.as_sk, pr.ws != nullptr, pr.ws_bytes, cus,
+                              pr.a_rows != nullptr);
   const Plan& pl = rs.pl;
   // everything that can refuse the launch is checked before the first pre-pass kernel is enqueued
   if (rs.grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)rs.grid);
@@ -663,6 +670,13 @@ int run(const Problem& pr) {
     if (!pr.act_s || misaligned(pr.act_s, 4) || misaligned(pr.c, 8))
       return fail(DLB_ERR_ALIGNMENT, "out_s is NULL or misaligned, or out_q is not 8-byte aligned");
     if (pr.act_s_sm < 0 || pr.act_s_sk < 0 || pr.act_s_sg < 0) return fail(DLB_ERR_BAD_STRIDE, "negative out_s stride");
+    if (pr.a_rows) {
+      // 32-bit DMA offsets count from the first row of the source matrix; its scales are gathered by the re-layout pass
+      if (pr.mode != kContiguous || !rs.relayout || pr.a_src_rows <= 0 || pr.a_src_rows * pr.K >= (1ll << 32))
+        return fail(DLB_ERR_BAD_SHAPE, "gathered activation rows need a workspace for their scales and rows * K < 2^32 (rows=%lld K=%lld)",
+                    (long long)pr.a_src_rows, (long long)pr.K);
+      if (misaligned(pr.a_rows, 4)) return fail(DLB_ERR_ALIGNMENT, "a_row_index is misaligned");
+    }
   }
   if (pl.variant == kVarExact && ceil_div(pr.N, 64) > (1ll << 31) - 1) return fail(DLB_ERR_BAD_SHAPE, "N too large for the exact path");
 
@@ -694,6 +708,7 @@ int run(const Problem& pr) {
   ar.kb_per_split = rs.kb_per_split;
   ar.group_m = g_knob[kKnobGroupM] > 0 ? g_knob[kKnobGroupM] : 8;
   ar.out_f32 = pr.out_dtype == DLB_OUT_F32;
+  ar.a_rows = pr.a_rows;
   ar.act_s = pr.act_s;
   ar.act_s_gs = pr.act_s_sg;
   ar.act_s_sm = pr.act_s_sm;
@@ -730,7 +745,7 @@ int run(const Problem& pr) {
                      static_cast<unsigned>(pr.mode == kMasked ? groups : 1));
     hipLaunchKernelGGL(fp8_scale_transpose_kernel, tgrid, dim3(256), 0, pr.stream, pr.a_s, relaid, static_cast<int>(pr.rows),
                        static_cast<int>(kblocks), static_cast<int>(rs.rows_pad), pr.mode == kMasked ? pr.as_sg : 0, pr.as_sm,
-                       pr.as_sk);
+                       pr.as_sk, pr.a_rows);
     e = hipGetLastError();
     if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "scale re-layout launch failed: %s", hipGetErrorString(e));
     ar.a_s = relaid;
@@ -928,6 +943,26 @@ int dlb_fp8_gemm_grouped_contiguous_silu_quant(const void* a, const void* b, con
   return dlb::run(pr);
 }
 
+int dlb_fp8_gemm_grouped_contiguous_gather_silu_quant(const void* a, const void* b, const float* a_s, const float* b_s,
+                                                      void* out_q, float* out_s, const int32_t* m_indices,
+                                                      const int32_t* a_row_index, int64_t a_rows, int64_t M_sum, int64_t N,
+                                                      int64_t K, int32_t G, int64_t as_stride_m, int64_t as_stride_k,
+                                                      int64_t os_stride_m, int64_t os_stride_k, float eps, void* workspace,
+                                                      size_t workspace_bytes, void* stream) {
+  dlb::Problem pr{dlb::kContiguous, a, b, a_s, b_s, out_q, m_indices, M_sum, N, K, G, 0, as_stride_m, as_stride_k,
+                  DLB_OUT_BF16, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  pr.act = true;
+  pr.act_s = out_s;
+  pr.act_s_sm = os_stride_m;
+  pr.act_s_sk = os_stride_k;
+  pr.act_eps = eps;
+  pr.a_rows = a_row_index;
+  pr.a_src_rows = a_rows;
+  if (M_sum > 0 && N > 0 && G > 0 && !out_s) return dlb::fail(DLB_ERR_NULL_POINTER, "out_s is NULL");
+  if (M_sum > 0 && N > 0 && G > 0 && !a_row_index) return dlb::fail(DLB_ERR_NULL_POINTER, "a_row_index is NULL");
+  return dlb::run(pr);
+}
+
 int dlb_fp8_gemm_grouped_masked_silu_quant(const void* a, const void* b, const float* a_s, const float* b_s, void* out_q,
                                            float* out_s, const int32_t* masked_m, int32_t expected_m, int64_t M_max,
                                            int64_t N, int64_t K, int32_t G, int64_t as_stride_g, int64_t as_stride_m,
@@ -1072,7 +1107,7 @@ int dlb_scale_relayout(const float* src, float* dst, int64_t rows, int64_t kbloc
   const dim3 grid(static_cast<unsigned>(ceil_div(rows_pad, 32)), static_cast<unsigned>(ceil_div(kblocks, 32)), 1);
   hipLaunchKernelGGL(fp8_scale_transpose_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), src, dst,
                      static_cast<int>(rows), static_cast<int>(kblocks), static_cast<int>(rows_pad), static_cast<int64_t>(0),
-                     src_stride_m, src_stride_k);
+                     src_stride_m, src_stride_k, static_cast<const int32_t*>(nullptr));
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "scale_relayout launch failed: %s", hipGetErrorString(e));
   return DLB_OK;

@@ -157,14 +157,17 @@ size_t dlb_ep_scatter_workspace_bytes(int64_t tokens, int64_t topk, int64_t expe
   return dlb::scatter_ws_bytes(tokens, topk, experts);
 }
 
-int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x_scale, int64_t xs_stride_m,
-                   int64_t xs_stride_k, const void* recv_topk, int topk_dtype, int64_t topk_stride_m,
-                   int64_t topk_stride_k, const int32_t* num_recv_tokens_per_expert, void* expert_start_loc,
-                   int start_dtype, void* output_tensor, int64_t out_row_stride, float* output_tensor_scale,
-                   int64_t os_stride_m, int64_t os_stride_k, int32_t* m_indices, int64_t m_indices_len,
-                   void* output_index, int index_dtype, int64_t oi_stride_m, int64_t oi_stride_k, int64_t tokens,
-                   int64_t hidden, int64_t topk, int64_t experts, void* workspace, size_t workspace_bytes,
-                   void* stream) {
+namespace {
+
+// ep_scatter with its tables only (index_only: no row is moved, src_row names every destination row's token) or in full
+int scatter_impl(const void* recv_x, int64_t x_row_stride, const float* recv_x_scale, int64_t xs_stride_m,
+                 int64_t xs_stride_k, const void* recv_topk, int topk_dtype, int64_t topk_stride_m,
+                 int64_t topk_stride_k, const int32_t* num_recv_tokens_per_expert, void* expert_start_loc,
+                 int start_dtype, void* output_tensor, int64_t out_row_stride, float* output_tensor_scale,
+                 int64_t os_stride_m, int64_t os_stride_k, int32_t* m_indices, int64_t m_indices_len,
+                 void* output_index, int index_dtype, int64_t oi_stride_m, int64_t oi_stride_k, int64_t tokens,
+                 int64_t hidden, int64_t topk, int64_t experts, void* workspace, size_t workspace_bytes,
+                 void* stream, int32_t* src_row, bool index_only) {
   using namespace dlb;
   clear_error();
   if (bad_index_dtype(topk_dtype) || bad_index_dtype(start_dtype) || bad_index_dtype(index_dtype))
@@ -182,14 +185,19 @@ int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x
     return fail(DLB_ERR_NULL_POINTER, "num_recv_tokens_per_expert, expert_start_loc or m_indices is NULL");
   const bool has_entries = tokens > 0 && topk > 0;
   if (has_entries && (!recv_topk || !output_index)) return fail(DLB_ERR_NULL_POINTER, "recv_topk or output_index is NULL");
-  if (has_entries && hidden > 0 && (!recv_x || !recv_x_scale || !output_tensor || !output_tensor_scale))
-    return fail(DLB_ERR_NULL_POINTER, "recv_x, recv_x_scale, output_tensor or output_tensor_scale is NULL");
-  if (x_row_stride < hidden || out_row_stride < hidden)
-    return fail(DLB_ERR_BAD_STRIDE, "row strides (%lld, %lld) are smaller than hidden=%lld", (long long)x_row_stride,
-                (long long)out_row_stride, (long long)hidden);
-  if (has_entries && hidden > 0 &&
-      (misaligned(recv_x, 16) || misaligned(output_tensor, 16) || x_row_stride % 16 != 0 || out_row_stride % 16 != 0))
-    return fail(DLB_ERR_ALIGNMENT, "recv_x / output_tensor rows must be 16-byte aligned");
+  if (index_only) {
+    if (m_indices_len > 0 && !src_row) return fail(DLB_ERR_NULL_POINTER, "src_row is NULL");
+    if (tokens > (1ll << 31) - 1) return fail(DLB_ERR_BAD_SHAPE, "tokens=%lld does not fit the int32 row table", (long long)tokens);
+  } else {
+    if (has_entries && hidden > 0 && (!recv_x || !recv_x_scale || !output_tensor || !output_tensor_scale))
+      return fail(DLB_ERR_NULL_POINTER, "recv_x, recv_x_scale, output_tensor or output_tensor_scale is NULL");
+    if (x_row_stride < hidden || out_row_stride < hidden)
+      return fail(DLB_ERR_BAD_STRIDE, "row strides (%lld, %lld) are smaller than hidden=%lld", (long long)x_row_stride,
+                  (long long)out_row_stride, (long long)hidden);
+    if (has_entries && hidden > 0 &&
+        (misaligned(recv_x, 16) || misaligned(output_tensor, 16) || x_row_stride % 16 != 0 || out_row_stride % 16 != 0))
+      return fail(DLB_ERR_ALIGNMENT, "recv_x / output_tensor rows must be 16-byte aligned");
+  }
   const size_t need = scatter_ws_bytes(tokens, topk > 0 ? topk : 1, experts);
   if (!workspace || workspace_bytes < need)
     return fail(DLB_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
@@ -217,6 +225,8 @@ int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x
   a.H = static_cast<int>(hidden), a.E = static_cast<int>(experts), a.topk_n = static_cast<int>(topk > 0 ? topk : 1);
   a.nblocks = scatter_blocks(a.T, a.topk_n, &a.tokens_per_block);
   a.topk_is64 = topk_dtype == DLB_IDX_I64, a.start_is64 = start_dtype == DLB_IDX_I64, a.oi_is64 = index_dtype == DLB_IDX_I64;
+  a.src_row = src_row;
+  a.index_only = index_only;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(a.nblocks)), block(kPermuteThreads);
   a.fused_scan = static_cast<int64_t>(a.nblocks) * a.E <= kFusedScanMaxInts;
@@ -238,6 +248,32 @@ int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x
   }
   hipLaunchKernelGGL(ep_scatter_copy_kernel, grid, dim3(kCopyThreads), 0, st, a);
   return finish("ep_scatter (copy)");
+}
+
+}  // namespace
+
+int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x_scale, int64_t xs_stride_m,
+                   int64_t xs_stride_k, const void* recv_topk, int topk_dtype, int64_t topk_stride_m,
+                   int64_t topk_stride_k, const int32_t* num_recv_tokens_per_expert, void* expert_start_loc,
+                   int start_dtype, void* output_tensor, int64_t out_row_stride, float* output_tensor_scale,
+                   int64_t os_stride_m, int64_t os_stride_k, int32_t* m_indices, int64_t m_indices_len,
+                   void* output_index, int index_dtype, int64_t oi_stride_m, int64_t oi_stride_k, int64_t tokens,
+                   int64_t hidden, int64_t topk, int64_t experts, void* workspace, size_t workspace_bytes,
+                   void* stream) {
+  return scatter_impl(recv_x, x_row_stride, recv_x_scale, xs_stride_m, xs_stride_k, recv_topk, topk_dtype, topk_stride_m,
+                      topk_stride_k, num_recv_tokens_per_expert, expert_start_loc, start_dtype, output_tensor, out_row_stride,
+                      output_tensor_scale, os_stride_m, os_stride_k, m_indices, m_indices_len, output_index, index_dtype,
+                      oi_stride_m, oi_stride_k, tokens, hidden, topk, experts, workspace, workspace_bytes, stream, nullptr, false);
+}
+
+int dlb_ep_scatter_rows(const void* recv_topk, int topk_dtype, int64_t topk_stride_m, int64_t topk_stride_k,
+                        const int32_t* num_recv_tokens_per_expert, void* expert_start_loc, int start_dtype,
+                        int32_t* m_indices, int32_t* src_row, int64_t m_indices_len, void* output_index, int index_dtype,
+                        int64_t oi_stride_m, int64_t oi_stride_k, int64_t tokens, int64_t topk, int64_t experts,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  return scatter_impl(nullptr, 0, nullptr, 0, 0, recv_topk, topk_dtype, topk_stride_m, topk_stride_k, num_recv_tokens_per_expert,
+                      expert_start_loc, start_dtype, nullptr, 0, nullptr, 0, 0, m_indices, m_indices_len, output_index, index_dtype,
+                      oi_stride_m, oi_stride_k, tokens, 0, topk, experts, workspace, workspace_bytes, stream, src_row, true);
 }
 
 int dlb_ep_gather(const void* input, int in_dtype, int64_t in_row_stride, const void* recv_topk_ids, int topk_dtype,

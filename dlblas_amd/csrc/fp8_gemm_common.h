@@ -65,6 +65,7 @@ struct Args {
   int tlist_cap;         //   entries per list
   // kContigListAct / kMaskedAct: c is the e4m3 output [G][M][act_cols] with row stride act_q_stride (bytes);
   // N = 2 act_cols weight rows
+  const int32_t* a_rows; //   kContigListAct, or NULL: row r of the GEMM is row a_rows[r] of a (its scales arrive re-laid by r)
   float* act_s;          //   scales of the output, element (g, m, j) at [g * act_s_gs + m * act_s_sm + j * act_s_sk]
   int64_t act_s_gs, act_s_sm, act_s_sk;
   int64_t act_q_stride;

@@ -115,8 +115,10 @@ struct PipeCfg {
 // contiguous, so that the GEMM's per-K-step fetch of one scale per tile row is a handful of full cache lines
 // instead of one line per row.  32 x 32 tiles through LDS keep both sides coalesced.  (The reference does the same
 // re-layout before its grouped GEMMs, dlblas/kernels/quant_dequant.py:42-83.)
+// rows_map (or NULL): row r of the re-laid copy is row rows_map[r] of src.
 __global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* src, float* dst, int rows, int kblocks,
-                                                                  int rows_pad, int64_t s_g, int64_t s_m, int64_t s_k) {
+                                                                  int rows_pad, int64_t s_g, int64_t s_m, int64_t s_k,
+                                                                  const int32_t* rows_map) {
   __shared__ float tile[32][33];
   const int g = blockIdx.z;
   const int r0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
@@ -126,7 +128,9 @@ __global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* s
 #pragma unroll
   for (int i = 0; i < 32; i += 8) {
     const int r = r0 + ty + i, k = k0 + tx;
-    tile[ty + i][tx] = (r < rows && k < kblocks) ? in[static_cast<int64_t>(r) * s_m + static_cast<int64_t>(k) * s_k] : 0.f;
+    const bool live = r < rows && k < kblocks;
+    const int64_t sr = (live && rows_map != nullptr) ? max(rows_map[r], 0) : r;
+    tile[ty + i][tx] = live ? in[sr * s_m + static_cast<int64_t>(k) * s_k] : 0.f;
   }
   __syncthreads();
 #pragma unroll
@@ -236,7 +240,10 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     const int64_t esz = p.out_f32 ? 4 : 2;
     const bool sliced = MODE == kDense && p.splitk > 1;
     const int kb_first = sliced ? split * p.kb_per_split : 0;  // the host leaves no slice empty
-    const uint8_t* a_tile = p.a + static_cast<int64_t>(m0) * p.K + static_cast<int64_t>(kb_first) * kScaleBlock;
+    // activation rows named by a table (the fused gate/up kernel reading the tokens where they lie, instead of a copy
+    // sorted by expert): per-lane offsets then count from the first row of the matrix
+    const bool a_indirect = MODE == kContigListAct && p.a_rows != nullptr;
+    const uint8_t* a_tile = p.a + static_cast<int64_t>(a_indirect ? 0 : m0) * p.K + static_cast<int64_t>(kb_first) * kScaleBlock;
     const float* as_tile = p.a_s + static_cast<int64_t>(m0) * p.as_sm + static_cast<int64_t>(kb_first) * p.as_sk;
     char* c_base = static_cast<char*>(p.c);
     if (kMaskedLike) {
@@ -270,8 +277,10 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     // barrier by every wave at once, kept the matrix pipe waiting).
     uint32_t a_off[Cfg::A_INST], b_off[Cfg::B_INST], s_off[Cfg::S_INST];
 #pragma unroll
-    for (int j = 0; j < Cfg::A_INST; ++j)
-      a_off[j] = static_cast<uint32_t>(min(dma_row + 8 * j * WAVES, a_last)) * uK + dma_chunk;
+    for (int j = 0; j < Cfg::A_INST; ++j) {
+      const int r = min(dma_row + 8 * j * WAVES, a_last);
+      a_off[j] = static_cast<uint32_t>(a_indirect ? max(p.a_rows[m0 + r], 0) : r) * uK + dma_chunk;
+    }
 #pragma unroll
     for (int j = 0; j < Cfg::B_INST; ++j)
       b_off[j] = static_cast<uint32_t>(kAct ? w_row(dma_row + 8 * j * WAVES) : min(dma_row + 8 * j * WAVES, b_last)) * uK + dma_chunk;

@@ -45,6 +45,8 @@ struct ScatterArgs {
   int H, E, topk_n, tokens_per_block, nblocks;
   int topk_is64, start_is64, oi_is64;
   int fused_scan;  // the copy kernel derives the block's first rows from the raw histograms itself (no scan launch)
+  int32_t* src_row;  // [m_len] or NULL: source token of every destination row (0 for rows nobody is copied to)
+  int index_only;    // fill the tables only: no row of x or xs is moved
 };
 
 // Expert id of entry `i` (token-major) of block `b`, or -1.
@@ -65,6 +67,12 @@ __global__ void __launch_bounds__(kPermuteThreads) ep_scatter_count_kernel(const
   if (id >= 0) atomicAdd(&hist[id], 1);
   __syncthreads();
   for (int e = threadIdx.x; e < p.E; e += kPermuteThreads) p.block_hist[static_cast<int64_t>(blockIdx.x) * p.E + e] = hist[e];
+  // rows that no slot is copied to (the padding of every expert's span) name token 0: any valid row will do for them,
+  // and this launch is ordered before the one that writes the real entries
+  if (p.src_row != nullptr)
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * kPermuteThreads + threadIdx.x; r < p.m_len;
+         r += static_cast<int64_t>(gridDim.x) * kPermuteThreads)
+      p.src_row[r] = 0;
 }
 
 // Pass 2 (one block of 1024): start_excl = exclusive prefix sum of counts; block_hist[b][e] becomes the first row
@@ -209,6 +217,7 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
       d = (p.fused_scan ? base_l[id] : static_cast<int64_t>(p.block_hist[static_cast<int64_t>(b) * p.E + id])) + rank;
       const int64_t t = static_cast<int64_t>(b) * p.tokens_per_block + tid / p.topk_n;
       store_index(p.out_index, p.oi_is64, t * p.oi_s0 + (tid % p.topk_n) * p.oi_s1, d);
+      if (p.src_row != nullptr && d < p.m_len) p.src_row[d] = static_cast<int32_t>(t);
     }
     dest[tid] = d;
   }
@@ -233,6 +242,7 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
     }
   }
 
+  if (p.index_only) return;
   // copies: one wave per token; a lane loads up to 8 chunks of 16 bytes (8 KB per wave and trip) before it stores
   // them to the row of every routed slot
   const int lane = tid & 63, wave = tid >> 6;

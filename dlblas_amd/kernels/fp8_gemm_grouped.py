@@ -86,12 +86,31 @@ def _(a, a_s, w, w_s, out_q, out_s, m_indices, eps):
     return True
 
 
-def fp8_gemm_grouped_contiguous_silu_quant(a, a_s, w13, w13_s, m_indices, eps: float = 1e-10, column_major_scales: bool = False):
+@torch.library.custom_op('dlblas::fp8_gemm_grouped_contiguous_gather_silu_quant', mutates_args=('out_q', 'out_s'),
+                         device_types='cuda')
+def grouped_contiguous_gather_silu_quant_op(a: torch.Tensor, a_s: torch.Tensor, w: torch.Tensor, w_s: torch.Tensor,
+                                            out_q: torch.Tensor, out_s: torch.Tensor, m_indices: torch.Tensor,
+                                            a_row_index: torch.Tensor, eps: float) -> bool:
+    G, N, K = w.shape
+    return _lib.gemm_contiguous_gather_silu_quant(a, w, a_s, w_s, out_q, out_s, m_indices, a_row_index, N, K, G, eps)
+
+
+@grouped_contiguous_gather_silu_quant_op.register_fake
+def _(a, a_s, w, w_s, out_q, out_s, m_indices, a_row_index, eps):
+    return True
+
+
+def fp8_gemm_grouped_contiguous_silu_quant(a, a_s, w13, w13_s, m_indices, eps: float = 1e-10, column_major_scales: bool = False,
+                                           a_row_index=None):
     """The first half of an expert MLP in one kernel: ``gate_up = grouped_contiguous(a, w13)`` (bf16), ``silu_and_mul``,
     ``per_token_group_quant_fp8(.., 128)`` - the sequence of dlblas/kernels/fused_moe_v3.py:307-334 with the same bits and
     without the bf16 intermediate in memory.  ``w13`` is [G, 2 I, K] with the gate rows first.  Returns (q e4m3fn
     [M_sum, I], s float32 [M_sum, I / 128]), or None when the library has no fused kernel for the shape (K or I not a
-    multiple of 128, ...): the caller then runs the three steps apart."""
+    multiple of 128, ...): the caller then runs the three steps apart.
+
+    ``a_row_index`` (int32 [M_sum], optional): row r of the GEMM is then row ``a_row_index[r]`` of ``a`` and ``a_s``, which
+    hold the tokens in the order they were received (``ep_scatter_rows`` writes the table), so that no expert-sorted copy
+    of the activations is needed."""
     for name, t, dt in (('a', a, torch.float8_e4m3fn), ('w13', w13, torch.float8_e4m3fn), ('a_s', a_s, torch.float32),
                         ('w13_s', w13_s, torch.float32)):
         if t.dtype != dt:
@@ -101,11 +120,14 @@ def fp8_gemm_grouped_contiguous_silu_quant(a, a_s, w13, w13_s, m_indices, eps: f
     if w13.dim() != 3 or a.dim() != 2 or a.size(1) != w13.size(2):
         raise ValueError(f'a must be [M_sum, K] and w13 [G, 2 I, K], got {tuple(a.shape)} and {tuple(w13.shape)}')
     G, N, K = w13.shape
-    M_sum = a.size(0)
+    M_sum = a.size(0) if a_row_index is None else m_indices.numel()
     if N % (2 * BLOCK) != 0 or K % BLOCK != 0:
         return None
-    if tuple(w13_s.shape) != (G, N // BLOCK, K // BLOCK) or tuple(a_s.shape) != (M_sum, K // BLOCK):
-        raise ValueError('a_s must be [M_sum, K / 128] and w13_s [G, 2 I / 128, K / 128]')
+    if tuple(w13_s.shape) != (G, N // BLOCK, K // BLOCK) or tuple(a_s.shape) != (a.size(0), K // BLOCK):
+        raise ValueError('a_s must be [rows of a, K / 128] and w13_s [G, 2 I / 128, K / 128]')
+    if a_row_index is not None and (a_row_index.dtype != torch.int32 or tuple(a_row_index.shape) != (M_sum, ) or
+                                    not a_row_index.is_contiguous()):
+        raise ValueError('a_row_index must be a contiguous int32 vector with one entry per GEMM row')
     if m_indices.dtype != torch.int32 or tuple(m_indices.shape) != (M_sum, ) or not m_indices.is_contiguous():
         raise ValueError('m_indices must be a contiguous int32 vector with one entry per row of a')
     inter = N // 2
@@ -115,6 +137,10 @@ def fp8_gemm_grouped_contiguous_silu_quant(a, a_s, w13, w13_s, m_indices, eps: f
     else:
         s = torch.empty((M_sum, inter // BLOCK), device=a.device, dtype=torch.float32)
     if M_sum == 0:
+        return q, s
+    if a_row_index is not None:
+        if a.size(0) == 0 or not grouped_contiguous_gather_silu_quant_op(a, a_s, w13, w13_s, q, s, m_indices, a_row_index, float(eps)):
+            return None
         return q, s
     if not grouped_contiguous_silu_quant_op(a, a_s, w13, w13_s, q, s, m_indices, float(eps)):
         return None

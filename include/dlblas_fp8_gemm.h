@@ -45,7 +45,7 @@
 extern "C" {
 #endif
 
-#define DLB_ABI_VERSION 4
+#define DLB_ABI_VERSION 5
 
 /* output element type of C */
 #define DLB_OUT_BF16 0
@@ -165,6 +165,29 @@ int dlb_fp8_gemm_grouped_contiguous_silu_quant(const void* a, const void* b, con
                                                int64_t as_stride_m, int64_t as_stride_k,
                                                int64_t os_stride_m, int64_t os_stride_k, float eps,
                                                void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * dlb_fp8_gemm_grouped_contiguous_silu_quant reading its activation rows where the tokens lie instead of from a copy
+ * sorted by expert: row r of the GEMM is row a_row_index[r] of a, and its scales are row a_row_index[r] of a_s.  With
+ * dlb_ep_scatter_rows (include/dlblas_fp8_moe.h), which fills m_indices, a_row_index and the slot table without moving
+ * a row, this replaces ep_scatter + the three steps of dlblas/kernels/fused_moe_v3.py:288-334; out_q / out_s hold the
+ * same bits as after the copy.
+ *
+ *   a            [a_rows, K]            e4m3fn, contiguous (the received tokens)
+ *   a_s          [a_rows, K/128]        fp32, element (t, kb) at a_s[t * as_stride_m + kb * as_stride_k]
+ *   a_row_index  [M_sum]                int32 on the device: source row of every GEMM row, 0 <= . < a_rows (rows of the
+ *                                       padding of an expert's span name any valid row; negative values are read as 0)
+ *   the other arguments as dlb_fp8_gemm_grouped_contiguous_silu_quant
+ *
+ * Needs what that entry point needs and a_rows * K < 2^32; otherwise DLB_ERR_BAD_SHAPE, nothing is enqueued.
+ */
+int dlb_fp8_gemm_grouped_contiguous_gather_silu_quant(const void* a, const void* b, const float* a_s, const float* b_s,
+                                                      void* out_q, float* out_s, const int32_t* m_indices,
+                                                      const int32_t* a_row_index, int64_t a_rows,
+                                                      int64_t M_sum, int64_t N, int64_t K, int32_t G,
+                                                      int64_t as_stride_m, int64_t as_stride_k,
+                                                      int64_t os_stride_m, int64_t os_stride_k, float eps,
+                                                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Grouped GEMM, fixed-capacity buffers with a valid-row count per expert.  Replaces

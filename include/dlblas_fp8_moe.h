@@ -97,6 +97,19 @@ int dlb_ep_scatter(const void* recv_x, int64_t x_row_stride, const float* recv_x
                    void* stream);
 
 /*
+ * The tables of dlb_ep_scatter without the copy: m_indices, expert_start_loc and output_index exactly as that call
+ * leaves them, plus src_row [m_indices_len] int32 = the token whose row dlb_ep_scatter would have copied to each
+ * destination row (0 for the rows of an expert's span that no slot is copied to).  No row of recv_x is read or written:
+ * dlb_fp8_gemm_grouped_contiguous_gather_silu_quant reads the tokens through src_row.  No counterpart in the
+ * reference, whose ep_scatter always copies (dlblas/kernels/fused_moe_v3.py:95-158).  Workspace as dlb_ep_scatter.
+ */
+int dlb_ep_scatter_rows(const void* recv_topk, int topk_dtype, int64_t topk_stride_m, int64_t topk_stride_k,
+                        const int32_t* num_recv_tokens_per_expert, void* expert_start_loc, int start_dtype,
+                        int32_t* m_indices, int32_t* src_row, int64_t m_indices_len, void* output_index, int index_dtype,
+                        int64_t oi_stride_m, int64_t oi_stride_k, int64_t tokens, int64_t topk, int64_t experts,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * out[t, :] = sum over the slots j with recv_topk_ids[t, j] >= 0, in slot order, of
  * input[input_index[t, j], :] * recv_topk_weight[t, j]; fp32 fused multiply-add chain, one cast at the end; a token
  * without a routed slot gets zeros.  Replaces ep_gather (dlblas/kernels/fused_moe_v3.py:199-233; kernel :161-196).

@@ -178,3 +178,57 @@ def test_masked_fused_full_size_and_low_latency_experts(dev):
     torch.cuda.synchronize()
     valid = torch.arange(M_max, device=dev)[None, :] < masked_m[:, None]
     assert torch.equal(out[valid], ref[valid])
+
+
+# --- the fused kernel reading the tokens through the row table of ep_scatter_rows (no expert-sorted copy) ------------
+
+
+@pytest.mark.parametrize('T,K,inter,E,topk,index_dtype', [
+    (96, 512, 256, 4, 2, torch.int64),
+    (700, 1024, 384, 8, 8, torch.int32),
+    (2000, 256, 128, 40, 3, torch.int64),
+])
+def test_gathered_rows_equal_the_copy(dev, T, K, inter, E, topk, index_dtype):
+    """ep_scatter_rows leaves the tables ep_scatter leaves, names the token of every destination row, and the fused
+    kernel that follows the table writes the bytes and scales of ep_scatter + the fused kernel on the copy."""
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_contiguous_silu_quant
+    from dlblas_amd.kernels.fused_moe_v3 import ep_scatter, ep_scatter_rows
+    print(f'case gathered fused gate/up T={T} K={K} I={inter} E={E} topk={topk}', flush=True)
+    g = helpers.gen(900 + T + K + E)
+    x_q, x_s = orc.quant_act_1x128((torch.randn(T, K, generator=g) * 1.5).to(torch.bfloat16))
+    ws = [orc.quant_weight_128x128((torch.randn(2 * inter, K, generator=g) * 0.05).to(torch.bfloat16)) for _ in range(E)]
+    w_q, w_s = torch.stack([w[0] for w in ws]).to(dev), torch.stack([w[1] for w in ws]).to(dev)
+    ids = torch.randint(-1, E, (T, topk), generator=g).to(index_dtype)
+    ids[torch.rand(T, topk, generator=g) < 0.3] = -1
+    routed = torch.bincount(ids[ids >= 0].long(), minlength=E)
+    counts = ((routed + 127) // 128 * 128).to(torch.int32).to(dev)
+    rows = int(counts.sum())
+    x_q, x_s, ids = x_q.to(dev), x_s.to(dev), ids.to(dev)
+
+    sorted_q = torch.zeros(rows, K, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    sorted_s = torch.ones(rows, K // 128, device=dev)
+    m_ref = torch.empty(rows, dtype=torch.int32, device=dev)
+    idx_ref = torch.full_like(ids, -1)
+    start_ref = torch.empty(E, dtype=torch.int64, device=dev)
+    ep_scatter(x_q, x_s, ids, counts, start_ref, sorted_q, sorted_s, m_ref, idx_ref)
+
+    m_got = torch.full((rows, ), -9, dtype=torch.int32, device=dev)
+    row_token = torch.full((rows, ), -9, dtype=torch.int32, device=dev)
+    idx_got = torch.full_like(ids, -1)
+    start_got = torch.empty(E, dtype=torch.int64, device=dev)
+    ep_scatter_rows(ids, counts, start_got, m_got, row_token, idx_got)
+    torch.cuda.synchronize()
+    assert torch.equal(m_got, m_ref) and torch.equal(idx_got, idx_ref) and torch.equal(start_got, start_ref)
+    valid = ids >= 0
+    tok = torch.arange(T, device=dev).unsqueeze(1).expand(T, topk)[valid]
+    assert torch.equal(row_token[idx_ref[valid]].long(), tok)
+    used = torch.zeros(rows, dtype=torch.bool, device=dev)
+    used[idx_ref[valid]] = True
+    assert (row_token[~used] == 0).all()
+
+    ref = fp8_gemm_grouped_contiguous_silu_quant(sorted_q, sorted_s, w_q, w_s, m_ref)
+    got = fp8_gemm_grouped_contiguous_silu_quant(x_q, x_s, w_q, w_s, m_got, a_row_index=row_token, column_major_scales=True)
+    torch.cuda.synchronize()
+    assert ref is not None and got is not None
+    assert torch.equal(got[0].view(torch.uint8)[used], ref[0].view(torch.uint8)[used]), 'quantised codes differ'
+    assert torch.equal(got[1][used], ref[1][used]), 'scales differ'
