@@ -636,7 +636,7 @@ def fused_moe_workload(dev):
     flops = 2.0 * n_routed * (2 * I * H + H * I)
     out = [{'workload': f'fused_moe_v3_T{T}_top{topk}_E{E}_H{H}_I{I}', 'routed_rows': n_routed, 'rows_padded': rows,
             'us_per_call': ms * 1e3, 'TFLOPs_on_routed_rows': flops / ms / 1e9,
-            'note': 'scatter, fused gate/up GEMM, down GEMM, gather with their pre-passes + per-call allocation of every intermediate, timed as one call of the Python driver'}]
+            'note': 'row tables, fused gate/up GEMM on the unsorted tokens, down GEMM, gather with their pre-passes + per-call allocation of every intermediate, timed as one call of the Python driver'}]
     # the decode counterpart: the masked expert MLP (dlblas_amd.kernels.moe.low_latency_experts) on 32 experts x 256
     # row slots with masked_m uniform in [0, 256]: fused gate/up GEMM + activation + quantiser, then the down GEMM
     from dlblas_amd.kernels.moe import low_latency_experts
