@@ -728,7 +728,27 @@ int run(const Problem& pr) {
   // workspace data region: [tile list][re-laid scales][partial sums of the K slices]
   size_t ws_used = 0;
   const bool tile_list = rs.tile_list;
-  if (tile_list) {
+  const bool one_prepass = tile_list && rs.relayout && pr.mode == kContiguous;
+  if (one_prepass) {
+    // tile list and scale re-layout in one launch
+    int32_t* tl = reinterpret_cast<int32_t*>(ar.ws);
+    ws_used = (static_cast<size_t>(2 + 2 * rs.nblk) * sizeof(int32_t) + 255) / 256 * 256;
+    float* relaid = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
+    const int tiles_x = static_cast<int>(ceil_div(rs.rows_pad, 32));
+    const dim3 pgrid(static_cast<unsigned>(tiles_x + 1), static_cast<unsigned>(ceil_div(kblocks, 32)), 1);
+    hipLaunchKernelGGL(contiguous_prepass_kernel, pgrid, dim3(256), 0, pr.stream, pr.gidx, static_cast<int>(pr.rows), pr.G, tl,
+                       static_cast<int>(rs.nblk), pr.a_s, relaid, static_cast<int>(kblocks), static_cast<int>(rs.rows_pad), pr.as_sm,
+                       pr.as_sk, pr.a_rows, tiles_x);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "pre-pass launch failed: %s", hipGetErrorString(e));
+    ar.tlist = tl;
+    ar.tlist_cap = static_cast<int>(rs.nblk);
+    ar.a_s = relaid;
+    ar.as_sm = 1;
+    ar.as_sk = rs.rows_pad;
+    ar.as_gs = kblocks * rs.rows_pad;
+  }
+  if (tile_list && !one_prepass) {
     // expert-contiguous rows: a device-built list of 256- and 128-row tiles (see contiguous_tile_list_kernel)
     int32_t* tl = reinterpret_cast<int32_t*>(ar.ws);
     hipLaunchKernelGGL(contiguous_tile_list_kernel, dim3(1), dim3(256), 0, pr.stream, pr.gidx, static_cast<int>(pr.rows), pr.G, tl,
@@ -739,7 +759,7 @@ int run(const Problem& pr) {
     ar.tlist_cap = static_cast<int>(rs.nblk);
     ws_used = (static_cast<size_t>(2 + 2 * rs.nblk) * sizeof(int32_t) + 255) / 256 * 256;
   }
-  if (rs.relayout) {
+  if (rs.relayout && !one_prepass) {
     float* relaid = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
     const dim3 tgrid(static_cast<unsigned>(ceil_div(rs.rows_pad, 32)), static_cast<unsigned>(ceil_div(kblocks, 32)),
                      static_cast<unsigned>(pr.mode == kMasked ? groups : 1));

@@ -115,13 +115,12 @@ struct PipeCfg {
 // contiguous, so that the GEMM's per-K-step fetch of one scale per tile row is a handful of full cache lines
 // instead of one line per row.  32 x 32 tiles through LDS keep both sides coalesced.  (The reference does the same
 // re-layout before its grouped GEMMs, dlblas/kernels/quant_dequant.py:42-83.)
-// rows_map (or NULL): row r of the re-laid copy is row rows_map[r] of src.
-__global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* src, float* dst, int rows, int kblocks,
-                                                                  int rows_pad, int64_t s_g, int64_t s_m, int64_t s_k,
-                                                                  const int32_t* rows_map) {
+// rows_map (or NULL): row r of the re-laid copy is row rows_map[r] of src.  (bx, by, g): the block's 32 x 32 tile and group.
+__device__ __forceinline__ void scale_transpose_block(const float* src, float* dst, int rows, int kblocks, int rows_pad,
+                                                      int64_t s_g, int64_t s_m, int64_t s_k, const int32_t* rows_map, int bx,
+                                                      int by, int g) {
   __shared__ float tile[32][33];
-  const int g = blockIdx.z;
-  const int r0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+  const int r0 = bx * 32, k0 = by * 32;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
   const float* in = src + static_cast<int64_t>(g) * s_g;
   float* out = dst + static_cast<int64_t>(g) * kblocks * rows_pad;
@@ -138,6 +137,12 @@ __global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* s
     const int k = k0 + ty + i, r = r0 + tx;
     if (k < kblocks && r < rows_pad) out[static_cast<int64_t>(k) * rows_pad + r] = tile[tx][ty + i];
   }
+}
+
+__global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* src, float* dst, int rows, int kblocks,
+                                                                  int rows_pad, int64_t s_g, int64_t s_m, int64_t s_k,
+                                                                  const int32_t* rows_map) {
+  scale_transpose_block(src, dst, rows, kblocks, rows_pad, s_g, s_m, s_k, rows_map, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
 // Work of one workgroup: tiles vb_first, vb_first + gridDim.x, ... of a region that is tiles_m x tiles_n tiles of
@@ -765,8 +770,7 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
 // not an expert) appear in no list.  list layout: [0] = n256, [1] = n128, [2 ..] 256-row list, [2 + cap ..] 128-row list.
 constexpr int kTileListMaxBlocks = 4096;  // 512 K rows; more rows fall back to uniform 128-row tiles
 
-__global__ void __launch_bounds__(256) contiguous_tile_list_kernel(const int32_t* m_indices, int M, int G, int32_t* tlist,
-                                                                   int cap) {
+__device__ __forceinline__ void contiguous_tile_list_block(const int32_t* m_indices, int M, int G, int32_t* tlist, int cap) {
   __shared__ int eb[kTileListMaxBlocks];   // expert of every 128-row block, -1 = skip
   __shared__ int rs[kTileListMaxBlocks];   // first block of the run of equal experts the block belongs to
   __shared__ int chunk_last[256];
@@ -801,6 +805,23 @@ __global__ void __launch_bounds__(256) contiguous_tile_list_kernel(const int32_t
   }
   __syncthreads();
   if (tid == 0) tlist[0] = n256, tlist[1] = n128;
+}
+
+__global__ void __launch_bounds__(256) contiguous_tile_list_kernel(const int32_t* m_indices, int M, int G, int32_t* tlist,
+                                                                   int cap) {
+  contiguous_tile_list_block(m_indices, M, G, tlist, cap);
+}
+
+// Both pre-passes of an expert-contiguous launch in one: the blocks of the scale re-layout, and one more column of
+// blocks (x == tiles_x) whose first builds the tile list.  One launch less in front of the GEMM (about 5 us).
+__global__ void __launch_bounds__(256) contiguous_prepass_kernel(const int32_t* m_indices, int M, int G, int32_t* tlist, int cap,
+                                                                 const float* src, float* dst, int kblocks, int rows_pad,
+                                                                 int64_t s_m, int64_t s_k, const int32_t* rows_map, int tiles_x) {
+  if (static_cast<int>(blockIdx.x) == tiles_x) {
+    if (blockIdx.y == 0) contiguous_tile_list_block(m_indices, M, G, tlist, cap);
+    return;
+  }
+  scale_transpose_block(src, dst, M, kblocks, rows_pad, 0, s_m, s_k, rows_map, blockIdx.x, blockIdx.y, 0);
 }
 
 template <class CfgA, class CfgB>
