@@ -246,7 +246,7 @@ int scatter_impl(const void* recv_x, int64_t x_row_stride, const float* recv_x_s
     hipLaunchKernelGGL(ep_scatter_scan_kernel, dim3(1), dim3(kScanThreads), kScanTileInts * 4, st, a);
     if (int rc = finish("ep_scatter (scan)")) return rc;
   }
-  hipLaunchKernelGGL(ep_scatter_copy_kernel, grid, dim3(kCopyThreads), 0, st, a);
+  hipLaunchKernelGGL(ep_scatter_copy_kernel, grid, dim3(index_only ? kPermuteThreads : kCopyThreads), 0, st, a);
   return finish("ep_scatter (copy)");
 }
 

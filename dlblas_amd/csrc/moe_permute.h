@@ -163,6 +163,7 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
   __shared__ int64_t base_l[kScanMaxExperts];      //             first row this block writes for every expert
   __shared__ int psum[kCopyThreads];
   const int tid = threadIdx.x;
+  const int nthreads = static_cast<int>(blockDim.x);  // kCopyThreads when rows are copied, kPermuteThreads for the tables only
   const int b = blockIdx.x;
   int id = -1;
   if (tid < kPermuteThreads) {
@@ -188,8 +189,8 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
       }
       if (tid == 0) excl_l[p.E] = carry;
     }
-    const int cols = min(p.E, kCopyThreads);
-    const int P = kCopyThreads / cols;
+    const int cols = min(p.E, nthreads);
+    const int P = nthreads / cols;
     const int my_part = tid / cols, my_col = tid % cols;
     for (int c0 = 0; c0 < p.E; c0 += cols) {
       const int e = c0 + my_col;
@@ -229,7 +230,7 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
     const int64_t total = min(excl[p.E], p.m_len);
     const int64_t per = (total + gridDim.x - 1) / gridDim.x;
     const int64_t r1 = min(total, (b + 1) * per);
-    for (int64_t r = b * per + tid; r < r1; r += kCopyThreads) {
+    for (int64_t r = b * per + tid; r < r1; r += nthreads) {
       int lo = 0, hi = p.E;  // largest e with start_excl[e] <= r
       while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -247,7 +248,7 @@ __global__ void __launch_bounds__(kCopyThreads) ep_scatter_copy_kernel(const Sca
   // them to the row of every routed slot
   const int lane = tid & 63, wave = tid >> 6;
   const int groups = p.H / 128;
-  for (int lt = wave; lt < p.tokens_per_block; lt += kCopyThreads / 64) {
+  for (int lt = wave; lt < p.tokens_per_block; lt += nthreads / 64) {
     const int64_t t = static_cast<int64_t>(b) * p.tokens_per_block + lt;
     if (t >= p.T) break;
     const uint8_t* src = p.x + t * p.x_row_stride;

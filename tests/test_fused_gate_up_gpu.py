@@ -187,6 +187,7 @@ def test_masked_fused_full_size_and_low_latency_experts(dev):
     (96, 512, 256, 4, 2, torch.int64),
     (700, 1024, 384, 8, 8, torch.int32),
     (2000, 256, 128, 40, 3, torch.int64),
+    (900, 128, 128, 300, 4, torch.int32),   # more experts than threads in a table-only block
 ])
 def test_gathered_rows_equal_the_copy(dev, T, K, inter, E, topk, index_dtype):
     """ep_scatter_rows leaves the tables ep_scatter leaves, names the token of every destination row, and the fused
