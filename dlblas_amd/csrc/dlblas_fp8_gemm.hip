@@ -123,7 +123,16 @@ typedef TileCfg<64, 128, 2, 2> Tile64x128;
 typedef TileCfg<128, 64, 2, 2> Tile128x64;
 typedef PipeCfg<4, 2, 2, 4, 2, 2> Pipe256x256;  // 8 waves, wave tile 64 x 128
 typedef PipeCfg<4, 2, 2, 3, 2, 2> Pipe256x192;  // narrow tiles of the mixed-width launch
+typedef PipeCfg<2, 4, 3, 2, 2, 2> Pipe192x256;  // the two tiles of an expert's run of three 128-row blocks
+
+// bytes of the three tile lists of an expert-contiguous launch over nblk 128-row blocks
+constexpr size_t tile_list_bytes(int64_t nblk) {
+  return (static_cast<size_t>(kTileListHeader + 3 * nblk) * sizeof(int32_t) + 255) / 256 * 256;
+}
 typedef PipeCfg<2, 4, 2, 2, 3> Pipe128x256w8;  // 8 waves, wave tile 64 x 64
+constexpr int kListLds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES
+                             ? (Pipe256x256::LDS_BYTES > Pipe192x256::LDS_BYTES ? Pipe256x256::LDS_BYTES : Pipe192x256::LDS_BYTES)
+                             : (Pipe128x256w8::LDS_BYTES > Pipe192x256::LDS_BYTES ? Pipe128x256w8::LDS_BYTES : Pipe192x256::LDS_BYTES);
 // small tiles for problems with few of the large ones (M of a few hundred, or a narrow N): 4 waves, deep rings
 typedef PipeCfg<2, 2, 2, 2, 4, 2, true> Pipe128x128;  // wave tile 64 x 64, 4 stages of 34 KB
 typedef PipeCfg<2, 2, 2, 1, 5, 2, true> Pipe128x64;   // wave tile 64 x 32, 5 stages of 26 KB
@@ -529,7 +538,7 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
   r.n_split = N;
   if (mode == kContiguous && pl.variant == kVarPipe128x256w8 && g_forced_variant < 0 && usable_ws && kblocks > 0) {
     const int64_t nblk = ceil_div(rows, kScaleBlock);
-    const size_t bytes = (static_cast<size_t>(2 + 2 * nblk) * sizeof(int32_t) + 255) / 256 * 256;
+    const size_t bytes = tile_list_bytes(nblk);
     if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
   }
   // gather_scales: the re-layout pass also brings the rows into the GEMM's order, so it runs whatever the strides
@@ -732,7 +741,7 @@ int run(const Problem& pr) {
   if (one_prepass) {
     // tile list and scale re-layout in one launch
     int32_t* tl = reinterpret_cast<int32_t*>(ar.ws);
-    ws_used = (static_cast<size_t>(2 + 2 * rs.nblk) * sizeof(int32_t) + 255) / 256 * 256;
+    ws_used = tile_list_bytes(rs.nblk);
     float* relaid = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
     const int tiles_x = static_cast<int>(ceil_div(rs.rows_pad, 32));
     const dim3 pgrid(static_cast<unsigned>(tiles_x + 1), static_cast<unsigned>(ceil_div(kblocks, 32)), 1);
@@ -757,7 +766,7 @@ int run(const Problem& pr) {
     if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "tile list launch failed: %s", hipGetErrorString(e));
     ar.tlist = tl;
     ar.tlist_cap = static_cast<int>(rs.nblk);
-    ws_used = (static_cast<size_t>(2 + 2 * rs.nblk) * sizeof(int32_t) + 255) / 256 * 256;
+    ws_used = tile_list_bytes(rs.nblk);
   }
   if (rs.relayout && !one_prepass) {
     float* relaid = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + ws_used);
@@ -820,8 +829,8 @@ int run(const Problem& pr) {
         e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
       else if (pl.variant == kVarPipe128x256w8 && tile_list && pr.act) {
         static std::atomic<unsigned long long> lds_done{0};
-        auto kernel = fp8_gemm_contig_list_act_kernel<Pipe256x256, Pipe128x256w8>;
-        constexpr int lds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES ? Pipe256x256::LDS_BYTES : Pipe128x256w8::LDS_BYTES;
+        auto kernel = fp8_gemm_contig_list_act_kernel<Pipe256x256, Pipe192x256, Pipe128x256w8>;
+        constexpr int lds = kListLds;
         e = ensure_lds(kernel, lds, dev, &lds_done);
         if (e == hipSuccess) {
           ar.tiles_n = static_cast<int>(pr.N / 256);  // 128 output columns = 128 gate + 128 up weight rows per tile
@@ -830,8 +839,8 @@ int run(const Problem& pr) {
         }
       } else if (pl.variant == kVarPipe128x256w8 && tile_list) {
         static std::atomic<unsigned long long> lds_done{0};
-        auto kernel = fp8_gemm_contig_list_kernel<Pipe256x256, Pipe128x256w8>;
-        constexpr int lds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES ? Pipe256x256::LDS_BYTES : Pipe128x256w8::LDS_BYTES;
+        auto kernel = fp8_gemm_contig_list_kernel<Pipe256x256, Pipe192x256, Pipe128x256w8>;
+        constexpr int lds = kListLds;
         e = ensure_lds(kernel, lds, dev, &lds_done);
         if (e == hipSuccess) {
           ar.tiles_n = static_cast<int>(ceil_div(pr.N, 256));

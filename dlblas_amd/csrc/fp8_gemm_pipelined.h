@@ -145,6 +145,8 @@ __global__ void __launch_bounds__(256) fp8_scale_transpose_kernel(const float* s
   scale_transpose_block(src, dst, rows, kblocks, rows_pad, s_g, s_m, s_k, rows_map, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
+constexpr int kTileListHeader = 3;  // tile counts in front of the three tile lists of an expert-contiguous launch
+
 // Work of one workgroup: tiles vb_first, vb_first + gridDim.x, ... of a region that is tiles_m x tiles_n tiles of
 // BM x BN and starts at column n_base of the output.
 template <class Cfg, int MODE>
@@ -206,13 +208,23 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     } else if (kList) {
       // tiles of this height come from the list the pre-pass built: entry = first 128-row block of the tile.  The
       // column tiles of one row block are adjacent in the order, so they share the activation tile in L2.
-      const int cnt = p.tlist[BM == 256 ? 0 : 1];
+      static_assert(BM == 256 || BM == 192 || BM == 128, "tile heights of the three lists");
+      constexpr int kWhich = BM == 256 ? 0 : (BM == 192 ? 1 : 2);
+      const int cnt = p.tlist[kWhich];
       const int total = cnt * tiles_n;
       if (vb >= total) break;
       const int t = xcd_remap(vb, total);
-      const int li = t / tiles_n;
-      nt = t - li * tiles_n;
-      m_first = p.tlist[2 + (BM == 256 ? 0 : p.tlist_cap) + li] * 128;
+      int li;
+      if (BM == 192) {
+        // the two tiles of a pair side by side for every column tile: neighbours in the order run on one XCD at the same time
+        const int pair = t / (2 * tiles_n), r = t - pair * 2 * tiles_n;
+        nt = r >> 1;
+        li = 2 * pair + (r & 1);
+      } else {
+        li = t / tiles_n;
+        nt = t - li * tiles_n;
+      }
+      m_first = p.tlist[kTileListHeader + kWhich * p.tlist_cap + li] * 64;
       g = p.gidx[m_first];
       m_end = min(p.M, m_first + BM);
     } else {
@@ -764,20 +776,25 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_pipelined_kernel(const Args 
 // one workgroup per tile, region A first.  The host picks the cut so that the last round of workgroups fills the
 // chip: e.g. 448 tiles of 256 x 256 on 256 CUs leave a quarter of the chip idle in the second round, while 256
 // tiles of 256 x 256 followed by 256 tiles of 256 x 192 cover the same output and keep every CU busy.
-// Expert-contiguous rows: a one-block pre-pass turns m_indices into two tile lists - 256-row tiles for pairs of
-// adjacent 128-row blocks of the same expert, 128-row tiles for what is left of every expert's run - so that most
-// weight tiles are fetched once per expert instead of once per 128 rows.  Blocks whose first index is negative (or
-// not an expert) appear in no list.  list layout: [0] = n256, [1] = n128, [2 ..] 256-row list, [2 + cap ..] 128-row list.
+// Expert-contiguous rows: a one-block pre-pass turns m_indices into three tile lists.  A run of R adjacent 128-row
+// blocks of one expert becomes R / 2 tiles of 256 rows when R is even, one tile of 128 rows when R = 1, and
+// (R - 3) / 2 tiles of 256 rows followed by two tiles of 192 rows when R is odd: most weight tiles are then fetched
+// once per expert instead of once per 128 rows, and the two 192-row tiles of an odd run, which are adjacent in their
+// list, run side by side on one XCD at the same pace, so that the second finds the weight tile in the L2 (a 256-row
+// and a 128-row tile drift apart and stream it twice).  Blocks whose first index is negative (or not an expert)
+// appear in no list.  list layout: [0] = n256, [1] = n192, [2] = n128, then the three lists of `cap` entries each;
+// an entry is the tile's first row in units of 64 rows.
 constexpr int kTileListMaxBlocks = 4096;  // 512 K rows; more rows fall back to uniform 128-row tiles
 
 __device__ __forceinline__ void contiguous_tile_list_block(const int32_t* m_indices, int M, int G, int32_t* tlist, int cap) {
   __shared__ int eb[kTileListMaxBlocks];   // expert of every 128-row block, -1 = skip
   __shared__ int rs[kTileListMaxBlocks];   // first block of the run of equal experts the block belongs to
-  __shared__ int chunk_last[256];
-  __shared__ int n256, n128;
+  __shared__ int re[kTileListMaxBlocks];   // last block of that run
+  __shared__ int chunk_last[256], chunk_first[256];
+  __shared__ int n256, n192, n128;
   const int tid = threadIdx.x;
   const int nblk = (M + 127) / 128;
-  if (tid == 0) n256 = n128 = 0;
+  if (tid == 0) n256 = n192 = n128 = 0;
   for (int b = tid; b < nblk; b += 256) {
     const int e = m_indices[static_cast<int64_t>(b) * 128];
     eb[b] = (e >= 0 && e < G) ? e : -1;
@@ -791,20 +808,49 @@ __device__ __forceinline__ void contiguous_tile_list_block(const int32_t* m_indi
     rs[b] = last;
   }
   chunk_last[tid] = last;
+  int first = nblk;  // the same from the right: nearest run end at or after the block
+  for (int b = b1 - 1; b >= b0; --b) {
+    if (b == nblk - 1 || eb[b] != eb[b + 1]) first = b;
+    re[b] = first;
+  }
+  chunk_first[tid] = first;
   __syncthreads();
-  int carry = -1;
-  for (int q = 0; q < tid; ++q) carry = max(carry, chunk_last[q]);
+  // what the chunks before (after) this one carry in: running maximum of chunk_last from the left, running minimum of
+  // chunk_first from the right, as two scans over the 256 chunk values in eight steps
+  for (int off = 1; off < 256; off <<= 1) {
+    const int from_left = tid >= off ? chunk_last[tid - off] : -1;
+    const int from_right = tid + off < 256 ? chunk_first[tid + off] : nblk;
+    __syncthreads();
+    chunk_last[tid] = max(chunk_last[tid], from_left);
+    chunk_first[tid] = min(chunk_first[tid], from_right);
+    __syncthreads();
+  }
+  const int carry = tid > 0 ? chunk_last[tid - 1] : -1;
   for (int b = b0; b < b1 && rs[b] < 0; ++b) rs[b] = carry;
+  const int carry_r = tid < 255 ? chunk_first[tid + 1] : nblk;
+  for (int b = b1 - 1; b >= b0 && re[b] >= nblk; --b) re[b] = carry_r;
   __syncthreads();
+  int32_t* l256 = tlist + kTileListHeader;
+  int32_t* l192 = l256 + cap;
+  int32_t* l128 = l192 + cap;
   for (int b = tid; b < nblk; b += 256) {
-    if (eb[b] < 0 || ((b - rs[b]) & 1)) continue;  // odd position in its run: second half of a 256-row tile
-    if (b + 1 < nblk && eb[b + 1] == eb[b])
-      tlist[2 + atomicAdd(&n256, 1)] = b;
-    else
-      tlist[2 + cap + atomicAdd(&n128, 1)] = b;
+    if (eb[b] < 0) continue;
+    const int pos = b - rs[b], len = re[b] - rs[b] + 1;
+    const bool odd_tail = (len & 1) && len >= 3 && pos >= len - 3;  // the last three blocks of an odd run: two 192-row tiles
+    if (odd_tail) {
+      if (pos == len - 3) {
+        const int at = atomicAdd(&n192, 2);
+        l192[at] = 2 * b;
+        l192[at + 1] = 2 * b + 3;
+      }
+    } else if (len == 1) {
+      l128[atomicAdd(&n128, 1)] = 2 * b;
+    } else if (!(pos & 1)) {
+      l256[atomicAdd(&n256, 1)] = 2 * b;  // even position: first half of a 256-row tile
+    }
   }
   __syncthreads();
-  if (tid == 0) tlist[0] = n256, tlist[1] = n128;
+  if (tid == 0) tlist[0] = n256, tlist[1] = n192, tlist[2] = n128;
 }
 
 __global__ void __launch_bounds__(256) contiguous_tile_list_kernel(const int32_t* m_indices, int M, int G, int32_t* tlist,
@@ -824,28 +870,37 @@ __global__ void __launch_bounds__(256) contiguous_prepass_kernel(const int32_t* 
   scale_transpose_block(src, dst, M, kblocks, rows_pad, 0, s_m, s_k, rows_map, blockIdx.x, blockIdx.y, 0);
 }
 
-template <class CfgA, class CfgB>
+// First workgroup-order index of a list's tiles for this workgroup when the lists before it hold `before` tiles: the
+// round robin continues where they ended.
+__device__ __forceinline__ int continue_round_robin(int before) {
+  const int grid = static_cast<int>(gridDim.x);
+  return (static_cast<int>(blockIdx.x) + grid - before % grid) % grid;
+}
+
+template <class CfgA, class CfgC, class CfgB>
 __global__ void __launch_bounds__(CfgA::NT) fp8_gemm_contig_list_kernel(const Args p) {
-  static_assert(CfgA::NT == CfgB::NT && CfgA::BN == CfgB::BN, "both tile heights use the same workgroup shape and width");
+  static_assert(CfgA::NT == CfgB::NT && CfgA::NT == CfgC::NT && CfgA::BN == CfgB::BN && CfgA::BN == CfgC::BN,
+                "the tile heights use the same workgroup shape and width");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  // persistent workgroups: tall tiles first, then the short ones continue the round robin where the tall ones ended
+  // persistent workgroups: 256-row tiles first, then the 192-row pairs, then the 128-row tiles
   pipelined_body<CfgA, kContigList>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
-  const int total_a = p.tlist[0] * p.tiles_n;
-  const int first_b = (static_cast<int>(blockIdx.x) + gridDim.x - total_a % gridDim.x) % gridDim.x;
-  pipelined_body<CfgB, kContigList>(p, smem, first_b, 0, p.tiles_n, 0);
+  const int total_a = p.tlist[0] * p.tiles_n, total_c = p.tlist[1] * p.tiles_n;
+  pipelined_body<CfgC, kContigList>(p, smem, continue_round_robin(total_a), 0, p.tiles_n, 0);
+  pipelined_body<CfgB, kContigList>(p, smem, continue_round_robin(total_a + total_c), 0, p.tiles_n, 0);
 }
 
 // The gate/up projection of an expert MLP with the activation and the quantiser of its output fused into the epilogue
 // (dlblas/kernels/fused_moe_v3.py:307-334 as one kernel): weights [G][2 I][K] with the gate rows first, output
 // e4m3 [M][I] + scales [M][I / 128].  Same tile lists and schedule as fp8_gemm_contig_list_kernel; tiles_n = I / 128.
-template <class CfgA, class CfgB>
+template <class CfgA, class CfgC, class CfgB>
 __global__ void __launch_bounds__(CfgA::NT) fp8_gemm_contig_list_act_kernel(const Args p) {
-  static_assert(CfgA::NT == CfgB::NT && CfgA::BN == CfgB::BN, "both tile heights use the same workgroup shape and width");
+  static_assert(CfgA::NT == CfgB::NT && CfgA::NT == CfgC::NT && CfgA::BN == CfgB::BN && CfgA::BN == CfgC::BN,
+                "the tile heights use the same workgroup shape and width");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   pipelined_body<CfgA, kContigListAct>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
-  const int total_a = p.tlist[0] * p.tiles_n;
-  const int first_b = (static_cast<int>(blockIdx.x) + gridDim.x - total_a % gridDim.x) % gridDim.x;
-  pipelined_body<CfgB, kContigListAct>(p, smem, first_b, 0, p.tiles_n, 0);
+  const int total_a = p.tlist[0] * p.tiles_n, total_c = p.tlist[1] * p.tiles_n;
+  pipelined_body<CfgC, kContigListAct>(p, smem, continue_round_robin(total_a), 0, p.tiles_n, 0);
+  pipelined_body<CfgB, kContigListAct>(p, smem, continue_round_robin(total_a + total_c), 0, p.tiles_n, 0);
 }
 
 template <class CfgA, class CfgB>
