@@ -513,7 +513,7 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
 struct Resolved {
   Plan pl;
   int splitk, kb_per_split;  // K slices summed in a second pass (1 = none), K blocks per slice
-  bool tile_list;            // expert-contiguous rows: device-built list of 256- and 128-row tiles
+  bool tile_list;            // expert-contiguous rows: device-built lists of 256-, 192- and 128-row tiles
   int64_t nblk;              //   128-row blocks it covers
   bool relayout;             // activation scales re-laid rows-contiguous in the workspace first
   int64_t rows_pad;          //   rows per K block of the re-laid copy
@@ -758,7 +758,7 @@ int run(const Problem& pr) {
     ar.as_gs = kblocks * rs.rows_pad;
   }
   if (tile_list && !one_prepass) {
-    // expert-contiguous rows: a device-built list of 256- and 128-row tiles (see contiguous_tile_list_kernel)
+    // expert-contiguous rows: device-built lists of 256-, 192- and 128-row tiles (see contiguous_tile_list_block)
     int32_t* tl = reinterpret_cast<int32_t*>(ar.ws);
     hipLaunchKernelGGL(contiguous_tile_list_kernel, dim3(1), dim3(256), 0, pr.stream, pr.gidx, static_cast<int>(pr.rows), pr.G, tl,
                        static_cast<int>(rs.nblk));
