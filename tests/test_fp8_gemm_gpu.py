@@ -343,6 +343,32 @@ def test_grouped_contiguous_run_lengths(dev, variant):
     helpers.tolerance_check(out, ref, f'contiguous run lengths {variant}')
 
 
+def test_grouped_contiguous_many_blocks(dev):
+    """700 blocks of 128 rows: the device-side tile list then works in chunks of several blocks per thread, and runs of
+    1 to 7 blocks (256-row tiles, pairs of 192-row tiles for the odd ones, single 128-row tiles) cross the chunk
+    boundaries in every way.  Skipped blocks in between; the last block is short."""
+    print('case contiguous many blocks', flush=True)
+    from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_contiguous
+    G, N, K = 12, 256, 128
+    g = helpers.gen(31)
+    blocks = []
+    while len(blocks) < 700:
+        e = int(torch.randint(-1, G, (1, ), generator=g))
+        blocks += [e] * int(torch.randint(1, 8, (1, ), generator=g))
+    blocks = blocks[:700]
+    M_sum = 128 * len(blocks) - 37
+    a_q, a_s = orc.quant_act_1x128(torch.randn(M_sum, K, generator=g).to(torch.bfloat16))
+    w_q, w_s = _make_grouped_weights(G, N, K, 32)
+    m_indices = torch.tensor(blocks, dtype=torch.int32).repeat_interleave(128)[:M_sum].contiguous()
+    sentinel = 99.0
+    ref = orc.grouped_contiguous_ref(a_q, a_s, w_q, w_s, torch.full((M_sum, N), sentinel), m_indices)
+    out = torch.full((M_sum, N), sentinel, dtype=torch.bfloat16, device=dev)
+    m_grouped_fp8_gemm_nt_contiguous((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, m_indices.to(dev))
+    torch.cuda.synchronize()
+    assert torch.all(out.cpu()[m_indices < 0] == sentinel), 'a skipped block was written'
+    helpers.tolerance_check(out, ref, 'contiguous many blocks')
+
+
 def test_grouped_masked(dev):
     print('case masked', flush=True)
     from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
