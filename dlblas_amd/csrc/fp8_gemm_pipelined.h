@@ -882,10 +882,12 @@ __global__ void __launch_bounds__(CfgA::NT) fp8_gemm_contig_list_kernel(const Ar
   static_assert(CfgA::NT == CfgB::NT && CfgA::NT == CfgC::NT && CfgA::BN == CfgB::BN && CfgA::BN == CfgC::BN,
                 "the tile heights use the same workgroup shape and width");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  // persistent workgroups: 256-row tiles first, then the 192-row pairs, then the 128-row tiles
-  pipelined_body<CfgA, kContigList>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
+  // persistent workgroups: the 192-row pairs first - every workgroup starts at the same moment, so the two tiles of a
+  // pair run in step from their first K block (2 - 4 % over starting them behind the 256-row tiles) - then the 256-row
+  // tiles, then the 128-row ones
   const int total_a = p.tlist[0] * p.tiles_n, total_c = p.tlist[1] * p.tiles_n;
-  pipelined_body<CfgC, kContigList>(p, smem, continue_round_robin(total_a), 0, p.tiles_n, 0);
+  pipelined_body<CfgC, kContigList>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
+  pipelined_body<CfgA, kContigList>(p, smem, continue_round_robin(total_c), 0, p.tiles_n, 0);
   pipelined_body<CfgB, kContigList>(p, smem, continue_round_robin(total_a + total_c), 0, p.tiles_n, 0);
 }
 
@@ -897,9 +899,9 @@ __global__ void __launch_bounds__(CfgA::NT) fp8_gemm_contig_list_act_kernel(cons
   static_assert(CfgA::NT == CfgB::NT && CfgA::NT == CfgC::NT && CfgA::BN == CfgB::BN && CfgA::BN == CfgC::BN,
                 "the tile heights use the same workgroup shape and width");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  pipelined_body<CfgA, kContigListAct>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
   const int total_a = p.tlist[0] * p.tiles_n, total_c = p.tlist[1] * p.tiles_n;
-  pipelined_body<CfgC, kContigListAct>(p, smem, continue_round_robin(total_a), 0, p.tiles_n, 0);
+  pipelined_body<CfgC, kContigListAct>(p, smem, blockIdx.x, 0, p.tiles_n, 0);
+  pipelined_body<CfgA, kContigListAct>(p, smem, continue_round_robin(total_c), 0, p.tiles_n, 0);
   pipelined_body<CfgB, kContigListAct>(p, smem, continue_round_robin(total_a + total_c), 0, p.tiles_n, 0);
 }
 
