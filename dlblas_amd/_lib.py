@@ -16,7 +16,9 @@ ABI_VERSION = 5
 OUT_BF16, OUT_F32 = 0, 1
 WS_COUNTER_BYTES = 65536
 WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
-STATIC_SCRATCH_BYTES = 16 << 20  # DLB_STATIC_SCRATCH_BYTES: the array dlb_fp8_gemm_noalloc works in
+STATIC_SCRATCH_BYTES = 16 << 20  # DLB_STATIC_SCRATCH_BYTES: the array dlb_fp8_gemm_noalloc works in ...
+STATIC_SCRATCH_SLICES = 4  # ... cut into this many slices, one per stream
+STATIC_SCRATCH_SLICE_BYTES = STATIC_SCRATCH_BYTES // STATIC_SCRATCH_SLICES
 
 ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_BAD_STRIDE, ERR_BAD_DTYPE, ERR_WORKSPACE, ERR_ALIGNMENT, ERR_LAUNCH = \
     -1, -2, -3, -4, -5, -6, -7
@@ -188,7 +190,8 @@ def force_variant(name_or_id) -> None:
     check(lib.dlb_fp8_gemm_force_variant(int(name_or_id)))
 
 
-KNOBS = {'splitk': 0, 'skinny_waves': 1, 'skinny_unroll': 2, 'skinny_nfrags': 3, 'group_m': 4, 'skinny_dma': 5, 'epilogue': 6, 'skinny_bn': 7}
+KNOBS = {'splitk': 0, 'skinny_waves': 1, 'skinny_unroll': 2, 'skinny_nfrags': 3, 'group_m': 4, 'skinny_dma': 5, 'epilogue': 6, 'skinny_bn': 7,
+         'splitk_mode': 8, 'spin_limit': 9, 'scale_table': 10, 'lds_oversize': 11}
 
 
 def tune(knob: str, value) -> None:

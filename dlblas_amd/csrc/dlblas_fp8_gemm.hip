@@ -93,9 +93,16 @@ enum Knob : int {
   kKnobSkinnyDma,  // 0 / 1: DMA-staged decode kernel where possible, 2: register-load decode kernel
   kKnobEpilogue,   // 0 / 1: bf16 output of the pipelined kernels goes through LDS where it can, 2: straight from registers
   kKnobSkinnyBn,   // columns per workgroup of the DMA-staged decode kernels (0 = heuristic)
+  kKnobSplitKMode, // 1: K slices of the ring kernels are added inside the launch where that applies; 0 / 2: by a second launch (faster on MI355X)
+  kKnobSpinLimit,  // one-launch split-K: value - 1 polls for the other slices of a tile (0 = default; 1 = none: the last arrival adds every share)
+  kKnobScaleTable, // 0 / 1: row-major activation scales of the small ring kernels go through the per-tile table, 2: never
+  kKnobLdsOversize,  // test hook: 1 = ask for more LDS than the GPU has, so that the launch is refused before anything is enqueued
   kKnobCount
 };
-thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0, 0};
+thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+// set while run() asks every kernel of the call for its launch attributes, before the first pre-pass is enqueued
+thread_local bool g_prepare_only = false;
+constexpr int kDefaultSpinLimit = 400;  // x about 0.5 us: far beyond the spread of the slices of one round of workgroups
 
 enum Variant : int {
   kVarExact = 0,
@@ -136,16 +143,29 @@ constexpr int kListLds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES
 // small tiles for problems with few of the large ones (M of a few hundred, or a narrow N): 4 waves, deep rings
 typedef PipeCfg<2, 2, 2, 2, 4, 2, true> Pipe128x128;  // wave tile 64 x 64, 4 stages of 34 KB
 typedef PipeCfg<2, 2, 2, 1, 5, 2, true> Pipe128x64;   // wave tile 64 x 32, 5 stages of 26 KB
+// the same with the activation scales of a tile in a table behind the ring (row-major a_s, at most 32 K blocks per workgroup)
+typedef PipeCfg<2, 2, 2, 2, 4, 2, true, true> Pipe128x128T;
+typedef PipeCfg<2, 2, 2, 1, 5, 2, true, true> Pipe128x64T;
+constexpr int kFusedMaxTiles = DLB_WS_COUNTER_BYTES / 16;  // four counter words per tile in the workspace head
 
 // Raise a kernel's dynamic LDS limit once per (kernel, device).
 template <class Kernel>
 hipError_t ensure_lds(Kernel kernel, int bytes, int dev, std::atomic<unsigned long long>* done_mask) {
+  if (g_knob[kKnobLdsOversize] == 1) {
+    const hipError_t e =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes + (1 << 20));
+    if (e != hipSuccess) (void)hipGetLastError();  // the refusal is reported through the return code, not left for the caller's next HIP call
+    return e;
+  }
   if (bytes <= 48 * 1024) return hipSuccess;
   const unsigned long long bit = 1ull << (dev & 63);
   if (done_mask->load(std::memory_order_acquire) & bit) return hipSuccess;
   const hipError_t e =
       hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (e == hipSuccess) done_mask->fetch_or(bit, std::memory_order_release);
+  if (e == hipSuccess)
+    done_mask->fetch_or(bit, std::memory_order_release);
+  else
+    (void)hipGetLastError();
   return e;
 }
 
@@ -154,7 +174,7 @@ hipError_t launch_tiled(const Args& args, int grid, int dev, hipStream_t stream)
   static std::atomic<unsigned long long> lds_done{0};
   auto kernel = fp8_gemm_tiled_kernel<Cfg, MODE>;
   hipError_t e = ensure_lds(kernel, Cfg::LDS_BYTES, dev, &lds_done);
-  if (e != hipSuccess) return e;
+  if (e != hipSuccess || g_prepare_only) return e;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
   return hipGetLastError();
 }
@@ -176,7 +196,7 @@ hipError_t launch_pipelined(const Args& args, int grid, int dev, hipStream_t str
   static std::atomic<unsigned long long> lds_done{0};
   auto kernel = fp8_gemm_pipelined_kernel<Cfg, MODE>;
   hipError_t e = ensure_lds(kernel, Cfg::LDS_BYTES, dev, &lds_done);
-  if (e != hipSuccess) return e;
+  if (e != hipSuccess || g_prepare_only) return e;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
   return hipGetLastError();
 }
@@ -201,14 +221,14 @@ hipError_t launch_skinny_cfg(bool dma, const Args& args, int dev, hipStream_t st
   if (dma && !ktail && Cfg::DMA_LDS_BYTES <= 160 * 1024 && g_knob[kKnobSkinnyDma] != 2) {
     auto kernel = fp8_gemm_skinny_dma_kernel<Cfg>;
     hipError_t e = ensure_lds(kernel, Cfg::DMA_LDS_BYTES, dev, &lds_done_dma);
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess || g_prepare_only) return e;
     const unsigned grid = static_cast<unsigned>(ceil_div(args.N, args.sk_bn));  // its own column split, see pick_skinny_bn
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NT), Cfg::DMA_LDS_BYTES, stream, args);
     return hipGetLastError();
   }
   auto kernel = ktail ? fp8_gemm_skinny_kernel<Cfg, true> : fp8_gemm_skinny_kernel<Cfg, false>;
   hipError_t e = ensure_lds(kernel, Cfg::RED_BYTES, dev, ktail ? &lds_done_tail : &lds_done);
-  if (e != hipSuccess) return e;
+  if (e != hipSuccess || g_prepare_only) return e;
   hipLaunchKernelGGL(kernel, dim3(args.tiles_n), dim3(Cfg::NT), Cfg::RED_BYTES, stream, args);
   return hipGetLastError();
 }
@@ -521,6 +541,9 @@ struct Resolved {
   int64_t n_split;           // mixed-width launch: first column of the 192-wide tiles (N: uniform 256-wide tiles)
   int64_t grid;              // workgroups of the main kernel
   bool resident;             // dense launch of many rounds: one resident workgroup per CU walks the tiles
+  bool sctab;                // small ring kernels: row-major activation scales through the per-tile table in LDS
+  int sct_shift;             //   log2 of the table's row pitch
+  bool fused;                // K slices added inside the launch (counters in the workspace head), no second pass
 };
 
 Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as_sm, int64_t as_sk, bool have_ws,
@@ -541,8 +564,15 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
     const size_t bytes = tile_list_bytes(nblk);
     if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
   }
+  // Small ring kernels with at most 32 K blocks per workgroup fetch a tile's row-major scales once, into a table in
+  // LDS: no re-layout pass, one cache-line request per row and tile.
+  const bool small_ring = pl.variant == kVarPipe128x128 || pl.variant == kVarPipe128x64;
+  auto table_fits = [&](int kb_per) {
+    return mode == kDense && small_ring && g_knob[kKnobScaleTable] != 2 && as_sm != 1 && kb_per <= 32 && as_sk < (1ll << 20) && dma_ok;
+  };
+  r.sctab = table_fits(r.kb_per_split);
   // gather_scales: the re-layout pass also brings the rows into the GEMM's order, so it runs whatever the strides
-  if (is_pipelined(pl.variant) && usable_ws &&
+  if (is_pipelined(pl.variant) && usable_ws && !r.sctab &&
       (gather_scales ? kblocks > 0 : as_sk == 1 && as_sm > 1 && kblocks > 1 && rows > kRelayoutMinRows)) {
     // row-major activation scales: re-lay them rows-contiguous in the workspace first (a few microseconds) so the
     // GEMM fetches 8 cache lines of scales per K step and tile instead of 256.  Up to 128 rows the extra launch costs
@@ -555,15 +585,26 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
     }
   }
   if (r.splitk > 1 && is_pipelined(pl.variant)) {
-    // the partial matrices of the K slices follow whatever else lives in the workspace; fewer slices if they do not fit
+    // One launch: the workgroups of a tile add its slices themselves.  Needs a single round of workgroups (they wait
+    // for each other, for a bounded time), a counter slot per tile and at most 32 slices (one claim bit each).
+    const int64_t tiles = ceil_div(rows, pl.bm) * ceil_div(N, pl.bn);
+    // Opt-in: on MI355X the device-scope round trips of that hand-over (stores out, counter, loads back) cost about
+    // 3 us more than ending the launch and starting a reduction kernel behind it.
+    r.fused = mode == kDense && g_knob[kKnobSplitKMode] == 1 && tiles <= kFusedMaxTiles && r.splitk <= 32 && tiles * r.splitk <= cus;
+    // the partial sums of the K slices follow whatever else lives in the workspace (whole tiles in the one-launch
+    // form, a [rows][N] matrix per slice otherwise); fewer slices if they do not fit
     const size_t avail = ws_bytes - DLB_WS_COUNTER_BYTES - r.ws_used;
-    const size_t per_slice = static_cast<size_t>(rows) * N * sizeof(float);
+    const size_t per_slice = r.fused ? static_cast<size_t>(tiles) * pl.bm * pl.bn * sizeof(float) : static_cast<size_t>(rows) * N * sizeof(float);
     if (per_slice * r.splitk > avail) {
       const int fit = per_slice > 0 && avail / per_slice >= 1 ? static_cast<int>(avail / per_slice) : 1;
       r.kb_per_split = static_cast<int>(ceil_div(kblocks, fit));
       r.splitk = static_cast<int>(ceil_div(kblocks, r.kb_per_split));
     }
+    if (r.splitk <= 1) r.fused = false;
   }
+  if (r.sctab && !table_fits(r.kb_per_split)) r.sctab = false;  // fewer, longer slices than the table holds: scales in place
+  if (r.sctab)
+    while ((1 << r.sct_shift) < r.kb_per_split) ++r.sct_shift;
   if (pl.variant == kVarPipe256mix) r.n_split = pick_mixed_split(rows, N, cus);
   const int64_t tiles_m = ceil_div(rows, pl.bm), tiles_n = ceil_div(N, pl.bn);
   int64_t grid = tiles_m * tiles_n * r.splitk;
@@ -725,8 +766,7 @@ int run(const Problem& pr) {
   ar.act_eps = pr.act_eps;
   ar.act_cols = static_cast<int>(pr.N / 2);
   ar.act_q_stride = pr.N / 2;
-  const size_t esz = ar.out_f32 ? 4 : 2;
-  ar.vec_store = (pr.N % 4 == 0) && !misaligned(pr.c, 4 * esz);
+  ar.vec_store = (pr.N % 4 == 0) && !misaligned(pr.c, 4 * (ar.out_f32 ? 4 : 2));
   ar.c_vec16 = !ar.out_f32 && pr.N % 8 == 0 && !misaligned(pr.c, 16) && g_knob[kKnobEpilogue] != 2;
   if (pr.ws && pr.ws_bytes >= DLB_WS_COUNTER_BYTES) {
     ar.ctr = static_cast<uint32_t*>(pr.ws);
@@ -734,9 +774,91 @@ int run(const Problem& pr) {
   }
 
   hipError_t e = hipSuccess;
+  ar.fused_reduce = rs.fused ? 1 : 0;
+  ar.spin_limit = g_knob[kKnobSpinLimit] > 0 ? g_knob[kKnobSpinLimit] - 1 : kDefaultSpinLimit;
+  ar.sct_shift = rs.sct_shift;
+  const bool tile_list = rs.tile_list;
+  const size_t esz = ar.out_f32 ? 4 : 2;
+
+  // The main kernel of the call.  With g_prepare_only set it only raises the kernel's dynamic-LDS limit (the one
+  // step of a launch that can still fail), so that run() can do that before it enqueues the first pre-pass.
+  auto main_kernel = [&]() -> hipError_t {
+    switch (pl.variant) {
+      case kVarExact: {
+        if (g_prepare_only) return hipSuccess;
+        // rows in a grid-stride loop: the second grid dimension is limited to 65535
+        const int64_t row_groups = ceil_div(pr.rows, 4);
+        const dim3 grid(static_cast<unsigned>(ceil_div(pr.N, 64)), static_cast<unsigned>(row_groups < 65535 ? row_groups : 65535));
+        hipLaunchKernelGGL(fp8_gemm_exact_kernel, grid, dim3(256), 0, pr.stream, ar);
+        return hipGetLastError();
+      }
+      case kVarSkinny16:
+        return launch_skinny(1, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
+      case kVarSkinny32:
+        return launch_skinny(2, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
+      case kVarSkinny64:
+        return launch_skinny(4, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
+      case kVarSkinny128:
+        return launch_skinny(8, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
+      default:
+        break;
+    }
+    const int g = static_cast<int>(rs.grid);
+    const int g_dense = rs.resident ? cus : g;
+    if (pl.variant == kVarPipe256mix) {
+      const int64_t split = rs.n_split;
+      if (split >= pr.N) return launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
+      static std::atomic<unsigned long long> lds_done{0};
+      auto kernel = fp8_gemm_pipelined_mixed_kernel<Pipe256x256, Pipe256x192>;
+      ar.n_split = static_cast<int>(split);
+      ar.tiles_n_a = static_cast<int>(split / 256);
+      ar.tiles_n_b = static_cast<int>(ceil_div(pr.N - split, 192));
+      ar.tiles_a = ar.tiles_m * ar.tiles_n_a;
+      const hipError_t le = ensure_lds(kernel, Pipe256x256::LDS_BYTES, dev, &lds_done);
+      if (le != hipSuccess || g_prepare_only) return le;
+      hipLaunchKernelGGL(kernel, dim3(ar.tiles_a + ar.tiles_m * ar.tiles_n_b), dim3(Pipe256x256::NT), Pipe256x256::LDS_BYTES,
+                         pr.stream, ar);
+      return hipGetLastError();
+    }
+    if (pl.variant == kVarPipe256x256) return launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
+    if (pl.variant == kVarPipe128x256w8 && tile_list && pr.act) {
+      static std::atomic<unsigned long long> lds_done{0};
+      auto kernel = fp8_gemm_contig_list_act_kernel<Pipe256x256, Pipe192x256, Pipe128x256w8>;
+      const hipError_t le = ensure_lds(kernel, kListLds, dev, &lds_done);
+      if (le != hipSuccess || g_prepare_only) return le;
+      ar.tiles_n = static_cast<int>(pr.N / 256);  // 128 output columns = 128 gate + 128 up weight rows per tile
+      hipLaunchKernelGGL(kernel, dim3(cus), dim3(Pipe256x256::NT), kListLds, pr.stream, ar);
+      return hipGetLastError();
+    }
+    if (pl.variant == kVarPipe128x256w8 && tile_list) {
+      static std::atomic<unsigned long long> lds_done{0};
+      auto kernel = fp8_gemm_contig_list_kernel<Pipe256x256, Pipe192x256, Pipe128x256w8>;
+      const hipError_t le = ensure_lds(kernel, kListLds, dev, &lds_done);
+      if (le != hipSuccess || g_prepare_only) return le;
+      ar.tiles_n = static_cast<int>(ceil_div(pr.N, 256));
+      hipLaunchKernelGGL(kernel, dim3(cus), dim3(Pipe256x256::NT), kListLds, pr.stream, ar);  // one resident workgroup per CU
+      return hipGetLastError();
+    }
+    if (pl.variant == kVarPipe128x256w8 && pr.act)
+      return launch_pipelined<Pipe128x256w8, kMaskedAct>(ar, g, dev, pr.stream);  // N / 256 column tiles, as the plain GEMM
+    if (pl.variant == kVarPipe128x256w8) return launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g_dense, dev, pr.stream);
+    if (pl.variant == kVarPipe128x128)
+      return rs.sctab ? launch_pipelined<Pipe128x128T, kDense>(ar, g, dev, pr.stream)
+                      : launch_pipelined_mode<Pipe128x128>(pr.mode, ar, g, dev, pr.stream);
+    if (pl.variant == kVarPipe128x64)
+      return rs.sctab ? launch_pipelined<Pipe128x64T, kDense>(ar, g, dev, pr.stream)
+                      : launch_pipelined_mode<Pipe128x64>(pr.mode, ar, g, dev, pr.stream);
+    if (pl.variant == kVarTile64x128) return launch_tiled_mode<Tile64x128>(pr.mode, ar, g, dev, pr.stream);
+    if (pl.variant == kVarTile128x64) return launch_tiled_mode<Tile128x64>(pr.mode, ar, g, dev, pr.stream);
+    return launch_tiled_mode<Tile128x128>(pr.mode, ar, g, dev, pr.stream);
+  };
+  g_prepare_only = true;
+  e = main_kernel();
+  g_prepare_only = false;
+  if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "the kernel's LDS size was refused, nothing enqueued: %s", hipGetErrorString(e));
+
   // workspace data region: [tile list][re-laid scales][partial sums of the K slices]
   size_t ws_used = 0;
-  const bool tile_list = rs.tile_list;
   const bool one_prepass = tile_list && rs.relayout && pr.mode == kContiguous;
   if (one_prepass) {
     // tile list and scale re-layout in one launch
@@ -783,88 +905,9 @@ int run(const Problem& pr) {
     ar.as_gs = kblocks * rs.rows_pad;
   }
   if (ar.splitk > 1 && is_pipelined(pl.variant)) ar.ws = reinterpret_cast<float*>(reinterpret_cast<char*>(ar.ws) + rs.ws_used);
-  switch (pl.variant) {
-    case kVarExact: {
-      // rows in a grid-stride loop: the second grid dimension is limited to 65535
-      const int64_t row_groups = ceil_div(pr.rows, 4);
-      const dim3 grid(static_cast<unsigned>(ceil_div(pr.N, 64)), static_cast<unsigned>(row_groups < 65535 ? row_groups : 65535));
-      hipLaunchKernelGGL(fp8_gemm_exact_kernel, grid, dim3(256), 0, pr.stream, ar);
-      e = hipGetLastError();
-      break;
-    }
-    case kVarSkinny16:
-      e = launch_skinny(1, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
-      break;
-    case kVarSkinny32:
-      e = launch_skinny(2, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
-      break;
-    case kVarSkinny64:
-      e = launch_skinny(4, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
-      break;
-    case kVarSkinny128:
-      e = launch_skinny(8, pl.sk_nfrags, pl.sk_waves, pl.sk_unroll, pl.sk_dma, ar, dev, pr.stream);
-      break;
-    default: {
-      const int g = static_cast<int>(rs.grid);
-      const int g_dense = rs.resident ? cus : g;
-      if (pl.variant == kVarPipe256mix) {
-        const int64_t split = rs.n_split;
-        if (split >= pr.N) {
-          e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
-        } else {
-          static std::atomic<unsigned long long> lds_done{0};
-          auto kernel = fp8_gemm_pipelined_mixed_kernel<Pipe256x256, Pipe256x192>;
-          ar.n_split = static_cast<int>(split);
-          ar.tiles_n_a = static_cast<int>(split / 256);
-          ar.tiles_n_b = static_cast<int>(ceil_div(pr.N - split, 192));
-          ar.tiles_a = ar.tiles_m * ar.tiles_n_a;
-          e = ensure_lds(kernel, Pipe256x256::LDS_BYTES, dev, &lds_done);
-          if (e == hipSuccess) {
-            hipLaunchKernelGGL(kernel, dim3(ar.tiles_a + ar.tiles_m * ar.tiles_n_b), dim3(Pipe256x256::NT),
-                               Pipe256x256::LDS_BYTES, pr.stream, ar);
-            e = hipGetLastError();
-          }
-        }
-      } else if (pl.variant == kVarPipe256x256)
-        e = launch_pipelined_mode<Pipe256x256>(pr.mode, ar, g_dense, dev, pr.stream);
-      else if (pl.variant == kVarPipe128x256w8 && tile_list && pr.act) {
-        static std::atomic<unsigned long long> lds_done{0};
-        auto kernel = fp8_gemm_contig_list_act_kernel<Pipe256x256, Pipe192x256, Pipe128x256w8>;
-        constexpr int lds = kListLds;
-        e = ensure_lds(kernel, lds, dev, &lds_done);
-        if (e == hipSuccess) {
-          ar.tiles_n = static_cast<int>(pr.N / 256);  // 128 output columns = 128 gate + 128 up weight rows per tile
-          hipLaunchKernelGGL(kernel, dim3(cus), dim3(Pipe256x256::NT), lds, pr.stream, ar);
-          e = hipGetLastError();
-        }
-      } else if (pl.variant == kVarPipe128x256w8 && tile_list) {
-        static std::atomic<unsigned long long> lds_done{0};
-        auto kernel = fp8_gemm_contig_list_kernel<Pipe256x256, Pipe192x256, Pipe128x256w8>;
-        constexpr int lds = kListLds;
-        e = ensure_lds(kernel, lds, dev, &lds_done);
-        if (e == hipSuccess) {
-          ar.tiles_n = static_cast<int>(ceil_div(pr.N, 256));
-          hipLaunchKernelGGL(kernel, dim3(cus), dim3(Pipe256x256::NT), lds, pr.stream, ar);  // one resident workgroup per CU
-          e = hipGetLastError();
-        }
-      } else if (pl.variant == kVarPipe128x256w8 && pr.act)
-        e = launch_pipelined<Pipe128x256w8, kMaskedAct>(ar, g, dev, pr.stream);  // N / 256 column tiles, as the plain GEMM
-      else if (pl.variant == kVarPipe128x256w8)
-        e = launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g_dense, dev, pr.stream);
-      else if (pl.variant == kVarPipe128x128)
-        e = launch_pipelined_mode<Pipe128x128>(pr.mode, ar, g, dev, pr.stream);
-      else if (pl.variant == kVarPipe128x64)
-        e = launch_pipelined_mode<Pipe128x64>(pr.mode, ar, g, dev, pr.stream);
-      else if (pl.variant == kVarTile64x128)
-        e = launch_tiled_mode<Tile64x128>(pr.mode, ar, g, dev, pr.stream);
-      else if (pl.variant == kVarTile128x64)
-        e = launch_tiled_mode<Tile128x64>(pr.mode, ar, g, dev, pr.stream);
-      else
-        e = launch_tiled_mode<Tile128x128>(pr.mode, ar, g, dev, pr.stream);
-    }
-  }
+  e = main_kernel();
   if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
-  if (ar.splitk > 1 && pr.mode == kDense && pl.variant != kVarExact && !is_skinny(pl.variant)) {
+  if (ar.splitk > 1 && !rs.fused && pr.mode == kDense && pl.variant != kVarExact && !is_skinny(pl.variant)) {
     const int64_t total = pr.rows * pr.N;
     const int vec_ok = total % 4 == 0 && !misaligned(pr.c, 4 * esz);
     hipLaunchKernelGGL(fp8_splitk_reduce_kernel, dim3(static_cast<unsigned>(ceil_div(ceil_div(total, 4), 256))), dim3(256), 0,
@@ -875,10 +918,14 @@ int run(const Problem& pr) {
   return DLB_OK;
 }
 
-// Device address of `scratch` on the current device, looked up once per device (with that device current) and kept.
-int static_scratch_ptr(void** out) {
+// The slice of `scratch` that calls on `stream` work in.  The array's device address is looked up once per device
+// (with that device current) and kept; a stream is bound to the first free slice of its device at its first call and
+// keeps it until the process ends, so calls on different streams never share scratch memory.  More streams than slices:
+// DLB_ERR_WORKSPACE.
+int static_scratch_slice(hipStream_t stream, void** out) {
   constexpr int kMaxDevices = 64;
   static std::atomic<void*> ptr_of[kMaxDevices];
+  static std::atomic<uintptr_t> owner[kMaxDevices][DLB_STATIC_SCRATCH_SLICES];  // 0 = free, else the stream handle + 1
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
   if (dev < 0 || dev >= kMaxDevices) return fail(DLB_ERR_LAUNCH, "device ordinal %d beyond the %d this library tracks", dev, kMaxDevices);
@@ -888,8 +935,18 @@ int static_scratch_ptr(void** out) {
     if (e != hipSuccess || !ptr) return fail(DLB_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
     ptr_of[dev].store(ptr, std::memory_order_release);
   }
-  *out = ptr;
-  return DLB_OK;
+  const uintptr_t key = reinterpret_cast<uintptr_t>(stream) + 1;
+  for (int i = 0; i < DLB_STATIC_SCRATCH_SLICES; ++i) {
+    uintptr_t cur = owner[dev][i].load(std::memory_order_acquire);
+    if (cur == 0 && owner[dev][i].compare_exchange_strong(cur, key, std::memory_order_acq_rel)) cur = key;
+    if (cur == key) {
+      *out = static_cast<char*>(ptr) + static_cast<size_t>(i) * DLB_STATIC_SCRATCH_SLICE_BYTES;
+      return DLB_OK;
+    }
+  }
+  return fail(DLB_ERR_WORKSPACE,
+              "the %d slices of the static scratch of device %d are bound to other streams; use dlb_fp8_gemm with a workspace "
+              "for this stream", DLB_STATIC_SCRATCH_SLICES, dev);
 }
 
 }  // namespace
@@ -931,19 +988,23 @@ int dlb_fp8_gemm_noalloc(const void* a, const void* b, const float* a_s, const f
   bool empty = false;
   const int bad = dlb::check_problem(pr, &empty);
   if (bad != DLB_OK || empty) return bad;
-  // the one hard requirement on the scratch: the activation scales, re-laid rows-contiguous, have to fit behind the
-  // reserved head (the K slices of the split-K plans adapt to whatever is left)
-  const int64_t relaid = dlb::ceil_div(K, dlb::kScaleBlock) * ((M + 3) / 4 * 4) * static_cast<int64_t>(sizeof(float));
-  if (relaid > static_cast<int64_t>(DLB_STATIC_SCRATCH_BYTES) - DLB_WS_COUNTER_BYTES - 256)
+  // What the plan of this problem would keep in a workspace of any size besides the partial sums of K slices (those
+  // adapt to the space there is): the activation scales re-laid rows-contiguous.  That has to fit a slice.
+  int dev = 0;
+  const int cus = dlb::device_cu_count(&dev);
+  if (cus < 0) return dlb::fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
+  const dlb::Resolved want = dlb::resolve(dlb::kDense, M, N, K, 1, as_stride_m, as_stride_k, true, static_cast<size_t>(1) << 40, cus);
+  const size_t room = DLB_STATIC_SCRATCH_SLICE_BYTES - DLB_WS_COUNTER_BYTES;
+  if (want.ws_used > room)
     return dlb::fail(DLB_ERR_WORKSPACE,
-                     "M=%lld x ceil(K/128)=%lld needs %lld bytes of re-laid scales, the static scratch holds %lld; use dlb_fp8_gemm "
-                     "with a workspace", (long long)M, (long long)dlb::ceil_div(K, dlb::kScaleBlock), (long long)relaid,
-                     (long long)(static_cast<int64_t>(DLB_STATIC_SCRATCH_BYTES) - DLB_WS_COUNTER_BYTES - 256));
+                     "M=%lld x ceil(K/128)=%lld needs %lld bytes of re-laid scales, a slice of the static scratch holds %lld; use "
+                     "dlb_fp8_gemm with a workspace", (long long)M, (long long)dlb::ceil_div(K, dlb::kScaleBlock), (long long)want.ws_used,
+                     (long long)room);
   void* ws = nullptr;
-  const int rc = dlb::static_scratch_ptr(&ws);
+  const int rc = dlb::static_scratch_slice(pr.stream, &ws);
   if (rc != DLB_OK) return rc;
   pr.ws = ws;
-  pr.ws_bytes = DLB_STATIC_SCRATCH_BYTES;
+  pr.ws_bytes = DLB_STATIC_SCRATCH_SLICE_BYTES;
   return dlb::run(pr);
 }
 

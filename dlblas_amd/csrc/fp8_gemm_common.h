@@ -34,7 +34,7 @@ struct Args {
   void* c;
   const int32_t* gidx;  // m_indices (contiguous) / masked_m (masked) / nullptr (dense)
   float* ws;            // scratch: split-K partial matrices [splitk][M][N]
-  uint32_t* ctr;        // reserved head of the workspace (unused)
+  uint32_t* ctr;        // head of the workspace: per-tile arrival / claim / exit counters of the one-launch split-K (all zero between launches)
   int64_t a_gs;         // per-expert strides in elements (masked mode)
   int64_t as_gs;
   int64_t c_gs;
@@ -53,6 +53,9 @@ struct Args {
   int sk_bn;            // decode kernels with DMA staging: output columns per workgroup (multiple of 4, <= 16 NFS)
   int splitk;
   int kb_per_split;
+  int fused_reduce;     // split-K in one launch: the workgroups of a tile add its K slices themselves (see splitk_fused_epilogue)
+  int spin_limit;       //   polls (about half a microsecond apart) a workgroup waits for the other slices of its tile before it leaves its share to the last one
+  int sct_shift;        // kernels with a scale table in LDS: log2 of the table's row pitch (a power of two >= K blocks per workgroup)
   int group_m;          // m-tiles per L2 swizzle group
   int out_f32;
   int vec_store;        // rows of c are aligned for 4-element vector stores

@@ -83,14 +83,34 @@ __device__ __forceinline__ void wait_vmcnt() {
 // for later stages stay in flight across it; the caller waits for the group it needs with wait_vmcnt first.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Four floats to / from memory that another workgroup of the same launch reads / wrote: device-scope accesses
+// (write-through, and read past the caches that are not coherent between the XCDs), 8 bytes each, relaxed.
+__device__ __forceinline__ void coherent_store16(float* dst, v4f v) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  uint64_t* d = reinterpret_cast<uint64_t*>(dst);
+  __hip_atomic_store(d, __builtin_bit_cast(uint64_t, v2f{v.x, v.y}), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(d + 1, __builtin_bit_cast(uint64_t, v2f{v.z, v.w}), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ v4f coherent_load16(const float* src) {
+  typedef float v2f __attribute__((ext_vector_type(2)));
+  const uint64_t* s = reinterpret_cast<const uint64_t*>(src);
+  const v2f lo = __builtin_bit_cast(v2f, __hip_atomic_load(s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  const v2f hi = __builtin_bit_cast(v2f, __hip_atomic_load(s + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  return v4f{lo.x, lo.y, hi.x, hi.y};
+}
+
 // PARTS_: 2 = the scale FMAs of a fragment run under the MFMAs of the NEXT fragment of the same wave (two partial
 // accumulators); 1 = they follow their own MFMAs and overlap with the other wave of the SIMD instead (16 fewer VGPRs).
 // PREFETCH_: true (one wave per SIMD, 512 registers) = every fragment of the NEXT K step is read into a second
 // register set while the current step computes, so no MFMA of a step waits for LDS.
-template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_, int PARTS_ = 2, bool PREFETCH_ = false>
+// SCTAB_: true = the activation scales of a tile's rows for ALL K blocks of the workgroup's K range (at most
+// SCTAB_KB) are fetched once per tile into a table behind the ring, lanes along K: a row-major a_s then costs one
+// cache-line request per row and tile instead of one per row and K step, and needs no re-layout pass in front.
+template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_, int PARTS_ = 2, bool PREFETCH_ = false, bool SCTAB_ = false>
 struct PipeCfg {
   static constexpr int WGM = WGM_, WGN = WGN_, MF = MF_, NF = NF_, STAGES = STAGES_, PARTS = PARTS_;
   static constexpr bool PREFETCH = PREFETCH_;
+  static constexpr bool SCTAB = SCTAB_;
   static constexpr bool UNIFORM_W = (128 % (NF_ * 32)) == 0;
   static constexpr int WAVES = WGM * WGN;
   static constexpr int NT = WAVES * 64;
@@ -98,13 +118,16 @@ struct PipeCfg {
   static constexpr int BN = WGN * NF * 32;
   static constexpr int A_INST = BM / 8 / WAVES;  // 16-byte DMA instructions per wave and stage for the A tile
   static constexpr int B_INST = BN / 8 / WAVES;
-  static constexpr int S_INST = (BM + NT - 1) / NT;  // 4-byte DMA instructions per wave for the a_s slice
+  static constexpr int S_INST = SCTAB ? 0 : (BM + NT - 1) / NT;  // 4-byte DMA instructions per wave for the a_s slice
   static constexpr int A_BYTES = BM * kScaleBlock;
   static constexpr int B_BYTES = BN * kScaleBlock;
   static constexpr int S_BYTES = S_INST * NT * 4;  // activation scales of the tile rows for one K block
   static constexpr int W_BYTES = NT * 4;           // weight scale of each wave's n block, one copy per lane
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + S_BYTES + W_BYTES;
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int SCTAB_KB = 32;              // K blocks per workgroup the table holds
+  static constexpr int SCTAB_OFF = STAGES * STAGE_BYTES;
+  static constexpr int SCTAB_BYTES = SCTAB ? BM * SCTAB_KB * 4 : 0;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + SCTAB_BYTES;
   static constexpr int LOADS_PER_STAGE = A_INST + B_INST + S_INST + 1;  // vmcnt units per wave and stage
   static_assert(BM % (8 * WAVES) == 0 && BN % (8 * WAVES) == 0, "tile rows must divide over the DMA instructions");
   static_assert(NF <= 4, "weight scales are fetched for at most four fragments per wave");
@@ -181,7 +204,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
   int walk_base = 0;
 
   for (int vb = vb_first;; vb += gridDim.x) {
-    int g = 0, mt = 0, nt, m_end, m_first = -1, split = 0;
+    int g = 0, mt = 0, nt, m_end, m_first = -1, split = 0, tile_lin = 0;
     if (kMaskedLike) {
       // The tile count is only known on the device, so the grid is persistent; the hardware deals consecutive
       // workgroups to the 8 XCDs in turn.  Of every 32 consecutive tiles each XCD takes 4 consecutive ones: the row
@@ -235,6 +258,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       const int id = xcd_remap(vb, units);
       split = MODE == kDense ? id / tiles : 0;
       const int t = id - split * tiles;
+      tile_lin = t;
       const int width = p.group_m * tiles_n;
       const int grp = t / width;
       const int first_m = grp * p.group_m;
@@ -257,6 +281,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     const int64_t esz = p.out_f32 ? 4 : 2;
     const bool sliced = MODE == kDense && p.splitk > 1;
     const int kb_first = sliced ? split * p.kb_per_split : 0;  // the host leaves no slice empty
+    const int nk = sliced ? min(p.kblocks, kb_first + p.kb_per_split) - kb_first : p.kblocks;  // K blocks of this unit
     // activation rows named by a table (the fused gate/up kernel reading the tokens where they lie, instead of a copy
     // sorted by expert): per-lane offsets then count from the first row of the matrix
     const bool a_indirect = MODE == kContigListAct && p.a_rows != nullptr;
@@ -292,7 +317,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     // Per-lane source offsets of every DMA instruction of a stage, computed once per tile: the K loop then issues
     // its DMA group without any vector ALU work (32-bit multiplies are quarter rate and, issued right behind the
     // barrier by every wave at once, kept the matrix pipe waiting).
-    uint32_t a_off[Cfg::A_INST], b_off[Cfg::B_INST], s_off[Cfg::S_INST];
+    uint32_t a_off[Cfg::A_INST], b_off[Cfg::B_INST], s_off[Cfg::S_INST > 0 ? Cfg::S_INST : 1];
 #pragma unroll
     for (int j = 0; j < Cfg::A_INST; ++j) {
       const int r = min(dma_row + 8 * j * WAVES, a_last);
@@ -382,13 +407,26 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
     constexpr int S = kHoldX ? NF : MF;        // streamed fragments
     constexpr int T = H * S;
     constexpr int kFragBytes = 32 * kScaleBlock;
-    const int nk = sliced ? min(p.kblocks, kb_first + p.kb_per_split) - kb_first : p.kblocks;  // K blocks of this unit
     const int held0 = (kHoldX ? wm0 : Cfg::BM + wn0) * kScaleBlock;      // byte offset of held fragment 0 in a stage
     const int strm0 = (kHoldX ? Cfg::BM + wn0 : wm0) * kScaleBlock;
     constexpr int kScaleOff = Cfg::A_BYTES + Cfg::B_BYTES;
     constexpr int kWScaleOff = kScaleOff + Cfg::S_BYTES;
 
     __syncthreads();  // the previous tile's readers and DMA groups are done with the ring
+    if constexpr (Cfg::SCTAB) {
+      // scale table [BM][1 << sct_shift]: entry (r, j) = a_s of tile row r at the workgroup's j-th K block.  One DMA
+      // instruction moves 64 consecutive entries, i.e. whole runs of a row's scales; issued ahead of the first stages,
+      // so the wait for stage 0 covers them.
+      const int shift = p.sct_shift;
+      const int n_inst = (BM << shift) >> 6;
+      for (int i = wave; i < n_inst; i += WAVES) {
+        const int e = i * 64 + lane;
+        const uint32_t r = static_cast<uint32_t>(min(e >> shift, a_last));
+        const uint32_t j = static_cast<uint32_t>(min(e & ((1 << shift) - 1), nk - 1));
+        dma_4(reinterpret_cast<const uint8_t*>(as_tile),
+              (r * static_cast<uint32_t>(p.as_sm) + j * static_cast<uint32_t>(p.as_sk)) * 4u, smem + Cfg::SCTAB_OFF + i * 256);
+      }
+    }
 #pragma unroll
     for (int s = 0; s < STAGES; ++s) issue_stage(min(s, nk - 1), s);
     if (STAGES >= 3)
@@ -409,16 +447,22 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       for (int u = 0; u < 16; ++u) part[0][u] = part[1][u] = 0.f;
       const int x0 = wm0 * kScaleBlock;
       const int w0 = (Cfg::BM + wn0) * kScaleBlock;
-      auto load_scales = [&](int base, float (&dst)[MF]) {
+      auto load_scales = [&](int base, int kbl, float (&dst)[MF]) {
         const float sb = *reinterpret_cast<const float*>(smem + base + kWScaleOff + wave * 256);
-        const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
+        if constexpr (Cfg::SCTAB) {
+          const float* tab = reinterpret_cast<const float*>(smem + Cfg::SCTAB_OFF);
 #pragma unroll
-        for (int mi = 0; mi < MF; ++mi) dst[mi] = sS[wm0 + mi * 32 + l32] * sb;
+          for (int mi = 0; mi < MF; ++mi) dst[mi] = tab[((wm0 + mi * 32 + l32) << p.sct_shift) + kbl] * sb;
+        } else {
+          const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
+#pragma unroll
+          for (int mi = 0; mi < MF; ++mi) dst[mi] = sS[wm0 + mi * 32 + l32] * sb;
+        }
       };
       // half-fragment q of a stage: q < 2 MF -> activation fragment q / 2, K half q % 2; else weight fragment
       constexpr int kHalves = 2 * (MF + NF);
       constexpr int kPerTile = (kHalves + (MF * NF) - 2) / (MF * NF - 1);  // spread over the first T - 1 tiles
-      load_scales(0, scb[0]);
+      load_scales(0, 0, scb[0]);
 #pragma unroll
       for (int mi = 0; mi < MF; ++mi) {
         xr[0][mi][0] = lds_read_frag32(smem, x0 + mi * kFragBytes, lc, 0);
@@ -451,7 +495,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
           z = mfma_32x32x64_e4m3(wr[B][ni][0], xr[B][mi][0], z);
           part[t & 1] = mfma_32x32x64_e4m3(wr[B][ni][1], xr[B][mi][1], z);
           __builtin_amdgcn_sched_barrier(0);
-          if (t == 0) load_scales(nxt_base, scb[B ^ 1]);
+          if (t == 0) load_scales(nxt_base, min(kb + 1, nk - 1), scb[B ^ 1]);
 #pragma unroll
           for (int q = t * kPerTile; q < (t + 1) * kPerTile && q < kHalves; ++q) {
             if (q < 2 * MF)
@@ -490,19 +534,20 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
 #pragma unroll
     for (int u = 0; u < 16; ++u) part[0][u] = part[1][u] = 0.f;
 
-    auto load_scales = [&](int base, float (&dst)[MF][NS]) {
+    auto load_scales = [&](int base, int kbl, float (&dst)[MF][NS]) {
       float sb[NS];
 #pragma unroll
       for (int j = 0; j < NS; ++j) sb[j] = *reinterpret_cast<const float*>(smem + base + kWScaleOff + wave * 256 + j * 4);
       const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
+      const float* tab = reinterpret_cast<const float*>(smem + Cfg::SCTAB_OFF);
 #pragma unroll
       for (int mi = 0; mi < MF; ++mi) {
-        const float sa = sS[wm0 + mi * 32 + l32];
+        const float sa = Cfg::SCTAB ? tab[((wm0 + mi * 32 + l32) << p.sct_shift) + kbl] : sS[wm0 + mi * 32 + l32];
 #pragma unroll
         for (int j = 0; j < NS; ++j) dst[mi][j] = sa * sb[j];
       }
     };
-    load_scales(0, sc);
+    load_scales(0, 0, sc);
 #pragma unroll
     for (int hi = 0; hi < H; ++hi) {
       hf[hi][0] = lds_read_frag32(smem, held0 + hi * kFragBytes, lc, 0);
@@ -578,7 +623,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         if (si == S - 1) {
           hf[hi][0] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 0);
           hf[hi][1] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 1);
-          if (hi == 0) load_scales(nxt_base, sc_next);
+          if (hi == 0) load_scales(nxt_base, min(kb + 1, nk - 1), sc_next);
           if (hi == H - 1) {
             sf[0] = lds_read_frag32(smem, nxt_base + strm0, lc, 0);
             sf[1] = lds_read_frag32(smem, nxt_base + strm0, lc, 1);
@@ -684,6 +729,119 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         if (row < BM && m < m_end) {
           *reinterpret_cast<v2i*>(q_out + static_cast<int64_t>(m) * p.act_q_stride + n0 + sub * 8) = v2i{packed[0], packed[1]};
           if (sub == 0) s_out[static_cast<int64_t>(m) * p.act_s_sm + static_cast<int64_t>(n0 / kScaleBlock) * p.act_s_sk] = scale;
+        }
+      }
+      continue;
+    }
+    if (sliced && p.fused_reduce) {
+      // Split-K in one launch.  The workgroups of a tile (one per K slice) park their fp32 sums in the workspace,
+      // count themselves in on the tile's arrival counter, wait - for a bounded time - until all slices are in, and
+      // then each adds up its share of the tile: the slices in index order (the same order, and so the same bits, as
+      // fp8_splitk_reduce_kernel), cast, store.  Nobody depends on that wait for correctness: a workgroup that gives
+      // up sets its bit in the tile's word of abandoned shares and looks at the counter once more (all in after all:
+      // it adds its share anyway); the workgroup whose arrival completed the tile reads that word after its own share
+      // and adds the shares named there.  A share that both of them add is stored twice with the same bits.  The last
+      // workgroup to leave the tile zeroes its three counters: the workspace head is all zero when the launch ends.
+      // Partial sums are written in accumulator order: unit ((wave MF + mi) NF + ni) 4 + u holds, for lane l, the four
+      // floats c[32 mi + (l & 31)][32 ni + 8 u + 4 (l >> 5) + 0..3] of that wave's tile.
+      constexpr int kTileFloats = BM * BN;
+      constexpr int kUnits = kTileFloats / 4;
+      const int S = p.splitk;
+      float* tbase = p.ws + static_cast<int64_t>(tile_lin) * S * kTileFloats;
+      float* mine = tbase + static_cast<int64_t>(split) * kTileFloats;
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NF; ++ni)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const v4f v = {acc[mi][ni][4 * u], acc[mi][ni][4 * u + 1], acc[mi][ni][4 * u + 2], acc[mi][ni][4 * u + 3]};
+            coherent_store16(mine + ((((wave * MF + mi) * NF + ni) * 4 + u) * 64 + lane) * 4, v);
+          }
+      // The stores above are write-through, device-scope stores: once the memory counter has drained they are where
+      // every XCD reads them.  (A release fence here would also write back the whole L2 of this XCD, once per
+      // workgroup: measured at 4 - 11 us per launch.)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();  // ... those of every wave; the ring is idle from here on
+      uint32_t* ctr = p.ctr + static_cast<int64_t>(tile_lin) * 4;
+      volatile uint32_t* flag = reinterpret_cast<volatile uint32_t*>(smem);
+      const uint32_t uS = static_cast<uint32_t>(S);
+      if (tid == 0) {
+        // the arrival and the first look at the counter travel together: one round trip instead of two
+        const uint32_t ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t seen = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = ticket + 1u == uS;
+        bool all_in = last || seen >= uS;
+#pragma unroll 1
+        for (int spin = 0; !all_in && spin < p.spin_limit; ++spin) {
+          __builtin_amdgcn_s_sleep(2);
+          all_in = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= uS;
+        }
+        if (!all_in) {
+          __hip_atomic_fetch_or(ctr + 1, 1u << split, __ATOMIC_SEQ_CST, __HIP_MEMORY_SCOPE_AGENT);
+          all_in = __hip_atomic_load(ctr, __ATOMIC_SEQ_CST, __HIP_MEMORY_SCOPE_AGENT) >= uS;
+        }
+        flag[0] = all_in ? 1u << split : 0u;
+        flag[1] = last ? 1u : 0u;
+      }
+      __syncthreads();
+      const bool last = flag[1] != 0;
+      const int64_t esz_c = p.out_f32 ? 4 : 2;
+      auto add_unit = [&](int u, const v4f& sum) {
+        const int ul = u & 63, uu = (u >> 6) & 3, f = u >> 8;  // f = (wave MF + mi) NF + ni
+        const int fni = f % NF, fmi = (f / NF) % MF, fw = f / (NF * MF);
+        const int m = m0 + (fw / Cfg::WGN) * (MF * 32) + fmi * 32 + (ul & 31);
+        const int n = n0 + (fw % Cfg::WGN) * (NF * 32) + fni * 32 + uu * 8 + (ul >> 5) * 4;
+        if (m >= m_end) return;
+        char* c_row = c_base + static_cast<int64_t>(m) * p.N * esz_c;
+        if (p.out_f32)
+          store_row4<true>(c_row, n, sum, p.N - n, p.vec_store);
+        else
+          store_row4<false>(c_row, n, sum, p.N - n, p.vec_store);
+      };
+      for (int round = 0; round < (last ? 2 : 1); ++round) {
+        if (round == 1) {
+          // the arrival that completed the tile, done with its own share: the shares their owners gave up on
+          __syncthreads();
+          if (tid == 0) flag[0] = __hip_atomic_load(ctr + 1, __ATOMIC_SEQ_CST, __HIP_MEMORY_SCOPE_AGENT);
+          __syncthreads();
+        }
+        const uint32_t todo = flag[0];
+        for (int j = 0; j < S; ++j) {
+          if (!((todo >> j) & 1u)) continue;
+          const int u0 = static_cast<int>(static_cast<int64_t>(j) * kUnits / S);
+          const int u1 = static_cast<int>(static_cast<int64_t>(j + 1) * kUnits / S);
+          // two units per thread and pass, the loads of up to eight slices of both in flight before the first sum
+          for (int ua = u0 + tid; ua < u1; ua += 2 * Cfg::NT) {
+            const int ub = ua + Cfg::NT;
+            const bool has_b = ub < u1;
+            v4f sum_a = {0.f, 0.f, 0.f, 0.f}, sum_b = {0.f, 0.f, 0.f, 0.f};
+            for (int sb = 0; sb < S; sb += 8) {
+              v4f pa[8], pb[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) {
+                pa[i] = pb[i] = v4f{0.f, 0.f, 0.f, 0.f};
+                if (sb + i < S) {
+                  pa[i] = coherent_load16(tbase + static_cast<int64_t>(sb + i) * kTileFloats + ua * 4);
+                  if (has_b) pb[i] = coherent_load16(tbase + static_cast<int64_t>(sb + i) * kTileFloats + ub * 4);
+                }
+              }
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                if (sb + i < S) sum_a += pa[i], sum_b += pb[i];
+            }
+            add_unit(ua, sum_a);
+            if (has_b) add_unit(ub, sum_b);
+          }
+        }
+      }
+      __syncthreads();  // flag[] is read; the next tile may use the ring
+      if (tid == 0) {
+        const uint32_t left = __hip_atomic_fetch_add(ctr + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left + 1u == uS) {
+          __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(ctr + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(ctr + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
       continue;

@@ -227,7 +227,13 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
 #pragma unroll
     for (int ni = 0; ni < NFS; ++ni) acc[mi][ni] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  for (int kb = wave; kb < nk; kb += WAVES * U) {
+  // One block in flight per wave (U == 1): the activation scales of FOUR consecutive blocks of the wave are fetched by
+  // one load per fragment - lane group q takes the block q rounds ahead - and handed to all lanes with a lane
+  // permute when their block comes up.  The four addresses of a row usually share a cache line (row-major a_s), so a
+  // wave asks for a quarter of the scale lines it would ask for block by block.
+  float sa_ahead[MF];
+  int it = 0;
+  for (int kb = wave; kb < nk; kb += WAVES * U, ++it) {
     float sa[U][MF], sb[U][NFS];
     // weights first: they are the HBM stream.  A K block past the end re-reads the last one with scale 0.
 #pragma unroll
@@ -259,8 +265,20 @@ __global__ void __launch_bounds__(Cfg::NT) fp8_gemm_skinny_dma_kernel(const Args
         const float v = bs_row[ni][kbu];
         sb[u][ni] = valid ? v : 0.f;
       }
+      if constexpr (U > 1) {
 #pragma unroll
-      for (int mi = 0; mi < MF; ++mi) sa[u][mi] = as_row[mi][static_cast<int64_t>(kbu) * p.as_sk];
+        for (int mi = 0; mi < MF; ++mi) sa[u][mi] = as_row[mi][static_cast<int64_t>(kbu) * p.as_sk];
+      }
+    }
+    if constexpr (U == 1) {
+      if ((it & 3) == 0) {
+        int kq = min(kb + q * WAVES, nk - 1) + rot;
+        kq = kq >= nk ? kq - nk : kq;
+#pragma unroll
+        for (int mi = 0; mi < MF; ++mi) sa_ahead[mi] = as_row[mi][static_cast<int64_t>(kq) * p.as_sk];
+      }
+#pragma unroll
+      for (int mi = 0; mi < MF; ++mi) sa[0][mi] = __shfl(sa_ahead[mi], ((it & 3) << 4) | l16);
     }
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): this wave's DMA groups have landed in its LDS area
 #pragma unroll

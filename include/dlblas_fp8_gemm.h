@@ -13,17 +13,18 @@
  *   - plain pointers and sizes only; every pointer is a DEVICE pointer unless stated otherwise;
  *   - the library never allocates, frees or synchronises; work is enqueued on `stream`
  *     (a hipStream_t passed as void*; NULL = the null stream) and the call returns at once;
- *   - return value 0 = enqueued, negative = rejected (see DLB_ERR_*), nothing was enqueued;
+ *   - return value 0 = enqueued, negative = rejected (see DLB_ERR_*), nothing was enqueued (every
+ *     check, and the one launch attribute that can be refused, comes before the first kernel of a call);
  *     dlb_last_error() gives a thread-local human-readable reason for the last failure;
  *   - no C++ exception ever crosses this boundary;
  *   - `workspace` is caller-owned device memory of at least dlb_fp8_gemm_workspace_bytes()
- *     bytes, 16-byte aligned.  Its first DLB_WS_COUNTER_BYTES bytes are reserved (no kernel
- *     of this version reads or writes them); the rest is scratch that a call overwrites:
- *     re-laid activation scales, fp32 partial sums of the split-K path, the tile list of the
- *     expert-contiguous path.  Nothing in it has
- *     to survive between calls, so one buffer serves any number of calls that do not overlap
- *     in time.  Two calls that may run concurrently (different streams) need separate
- *     workspaces.
+ *     bytes, 16-byte aligned.  Its first DLB_WS_COUNTER_BYTES bytes hold the counters of the
+ *     one-launch split-K path (DLB_KNOB_SPLITK_MODE): they must be ZERO before the first call
+ *     that uses the buffer, and every call leaves them zero.  The rest is scratch that a call
+ *     overwrites: re-laid activation scales, fp32 partial sums of the split-K path, the tile
+ *     list of the expert-contiguous path; nothing there has to be initialised or to survive
+ *     between calls, so one buffer serves any number of calls that do not overlap in time.
+ *     Two calls that may run concurrently (different streams) need separate workspaces.
  *
  * Reference interfaces these replace (paths relative to the DLBlas source tree):
  *   - dlb_fp8_gemm                     : dlblas/kernels/fp8_gemm.py:15-65 (kernel) and :68-89 (host wrapper)
@@ -99,19 +100,26 @@ int dlb_fp8_gemm(const void* a, const void* b, const float* a_s, const float* b_
  * dlb_fp8_gemm for callers that cannot allocate device memory and have no workspace to pass: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its Triton launch
  * needs no scratch).  Same operands, same kernels and same results as dlb_fp8_gemm called with a workspace of
- * DLB_STATIC_SCRATCH_BYTES bytes; the scratch (re-laid activation scales, fp32 partial sums of the split-K plans) is
- * a fixed array inside the library's code object, DLB_STATIC_SCRATCH_BYTES per GPU, held by every GPU the library
- * runs on until the process ends.  The call allocates and frees nothing and does not synchronise.
+ * DLB_STATIC_SCRATCH_SLICE_BYTES bytes; the scratch (re-laid activation scales, fp32 partial sums of the split-K
+ * plans) is a fixed array inside the library's code object, DLB_STATIC_SCRATCH_BYTES per GPU, held by every GPU the
+ * library runs on until the process ends.  The call allocates and frees nothing and does not synchronise.
  *
- *   - Limit: 4 * ceil(K/128) * M bytes (M rounded up to a multiple of 4) must fit in DLB_STATIC_SCRATCH_BYTES minus
- *     the reserved head (64 KiB + 256); larger problems are rejected with DLB_ERR_WORKSPACE and nothing is enqueued.
- *   - All calls on one GPU share that GPU's array and overwrite what the previous call left in it (nothing in it has
- *     to be zero at entry): calls that may overlap in time on one GPU - different streams - race; order them or use
- *     dlb_fp8_gemm with a workspace per stream.
+ *   - The array is cut into DLB_STATIC_SCRATCH_SLICES slices.  A stream is bound to the first free slice of its GPU at
+ *     its first call and keeps it until the process ends: calls on different streams never share scratch memory, calls
+ *     on one stream are ordered by the stream.  A call on one more stream than there are slices is rejected with
+ *     DLB_ERR_WORKSPACE (use dlb_fp8_gemm with a workspace of its own for that stream).
+ *   - Limit: what the plan keeps in scratch besides the partial sums (which adapt to the room there is) has to fit a
+ *     slice minus its 64 KiB head: the re-laid activation scales, 4 * ceil(K/128) * M bytes (M rounded up to a multiple
+ *     of 4), when M > 128 and a_s is row-major and the plan is not one of the small-tile ones that read a_s in place.
+ *     Larger problems are rejected with DLB_ERR_WORKSPACE and nothing is enqueued.
+ *   - A call overwrites what the previous call on its stream left in the slice; nothing in it has to be initialised
+ *     (the array is zero when the library is loaded and every call leaves the slice's head zero).
  *   - The first call on a device looks up the array's device address (hipGetSymbolAddress); make that call outside
  *     a graph capture.
  */
 #define DLB_STATIC_SCRATCH_BYTES (16u << 20)
+#define DLB_STATIC_SCRATCH_SLICES 4
+#define DLB_STATIC_SCRATCH_SLICE_BYTES (DLB_STATIC_SCRATCH_BYTES / DLB_STATIC_SCRATCH_SLICES)
 int dlb_fp8_gemm_noalloc(const void* a, const void* b, const float* a_s, const float* b_s, void* c,
                          int64_t M, int64_t N, int64_t K,
                          int64_t as_stride_m, int64_t as_stride_k,
@@ -307,6 +315,16 @@ int dlb_fp8_gemm_force_variant(int variant);
  *   DLB_KNOB_SKINNY_DMA     2 = decode kernels load operands through registers instead of the LDS DMA path
  *   DLB_KNOB_EPILOGUE       2 = the pipelined kernels store bf16 results straight from registers (no LDS transpose)
  *   DLB_KNOB_SKINNY_BN      output columns per workgroup of the DMA-staged decode kernels (multiple of 4, at most 32)
+ *   DLB_KNOB_SPLITK_MODE    1 = the K slices of the DMA-ring kernels are added inside the launch (one launch per call: the
+ *                           workgroups of a tile count themselves in on a counter in the workspace head and add the
+ *                           slices in index order, the same bits as the second pass); 0 / 2 = by a second launch, which
+ *                           is the faster of the two on MI355X
+ *   DLB_KNOB_SPIN_LIMIT     one-launch split-K: value - 1 = polls a workgroup waits for the other slices of its tile
+ *                           (1 = none: the workgroup that completes a tile adds all of it)
+ *   DLB_KNOB_SCALE_TABLE    2 = the small DMA-ring kernels fetch row-major activation scales stage by stage instead of
+ *                           once per tile into a table in LDS
+ *   DLB_KNOB_LDS_OVERSIZE   test hook: 1 = every kernel asks for more LDS than the GPU has, so the call is refused
+ *                           (DLB_ERR_LAUNCH) before anything is enqueued
  */
 #define DLB_KNOB_SPLITK 0
 #define DLB_KNOB_SKINNY_WAVES 1
@@ -316,6 +334,10 @@ int dlb_fp8_gemm_force_variant(int variant);
 #define DLB_KNOB_SKINNY_DMA 5
 #define DLB_KNOB_EPILOGUE 6
 #define DLB_KNOB_SKINNY_BN 7
+#define DLB_KNOB_SPLITK_MODE 8
+#define DLB_KNOB_SPIN_LIMIT 9
+#define DLB_KNOB_SCALE_TABLE 10
+#define DLB_KNOB_LDS_OVERSIZE 11
 int dlb_fp8_gemm_tune(int knob, int value);
 
 /* Name of kernel variant `variant`, or NULL beyond the last one. */

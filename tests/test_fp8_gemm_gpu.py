@@ -86,6 +86,86 @@ def test_split_k_two_pass(dev, M, N, K, variant, splitk, out_dtype):
     assert torch.equal(out, again)
 
 
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('variant,splitk', [('pipe128x64', 7), ('pipe128x64', 2), ('pipe128x128', 4), ('pipe128x128', 32), ('pipe128x256w8', 3),
+                                            ('pipe256x256', 5)])
+@pytest.mark.parametrize('M,N,K', [(128, 2112, 7168), (200, 392, 2048), (129, 130, 4096), (33, 64, 4096)])
+def test_split_k_in_one_launch_equals_two_pass(dev, M, N, K, variant, splitk, out_dtype):
+    """The K slices of a tile added by its own workgroups (arrival counter in the workspace head, bounded wait, slices
+    summed in index order) give the bits of the two-pass path; so does the path in which nobody waits and the workgroup
+    that completes a tile adds every share (spin limit 0).  Every call leaves the counter head all zero."""
+    from dlblas_amd import _lib
+    print(f'case one-launch split-K variant={variant} splitk={splitk} M={M} N={N} K={K} {out_dtype}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=13)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    head = _lib.workspace(dev, torch.cuda.current_stream().cuda_stream)[:_lib.WS_COUNTER_BYTES]
+    outs = []
+    try:
+        _lib.force_splitk(splitk)
+        for mode, spin in ((2, 0), (1, 0), (1, 1), (1, 0)):
+            _lib.tune('splitk_mode', mode)
+            _lib.tune('spin_limit', spin)
+            outs.append(_run_dense(dev, a_q, a_s, b_q, b_s, dtype=out_dtype, variant=variant))
+            assert int(head.count_nonzero()) == 0, f'counter head not zero after mode {mode} spin {spin}'
+    finally:
+        _lib.force_splitk(0)
+        _lib.tune('splitk_mode', 0)
+        _lib.tune('spin_limit', 0)
+    helpers.tolerance_check(outs[0], ref, f'one-launch split-K {variant}/{splitk} {M}x{N}x{K}')
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
+@pytest.mark.parametrize('variant,splitk', [('pipe128x64', 0), ('pipe128x64', 7), ('pipe128x128', 2), ('pipe128x128', 5)])
+@pytest.mark.parametrize('M,N,K', [(128, 2112, 7168), (256, 520, 2048), (77, 200, 4096), (300, 392, 1024)])
+def test_scale_table_equals_scales_per_stage(dev, M, N, K, variant, splitk):
+    """Row-major activation scales fetched once per tile into the table in LDS (the default of the small ring kernels up
+    to 32 K blocks per workgroup) against the same kernels fetching them stage by stage: the same values, the same bits.
+    Column-major scales never take the table."""
+    from dlblas_amd import _lib
+    print(f'case scale table variant={variant} splitk={splitk} M={M} N={N} K={K}', flush=True)
+    a_q, a_s, b_q, b_s = helpers.make_dense(M, N, K, seed=19)
+    ref = orc.dequant_ref(a_q, a_s, b_q, b_s)
+    try:
+        _lib.force_splitk(splitk)
+        with_table = _run_dense(dev, a_q, a_s, b_q, b_s, variant=variant)
+        _lib.tune('scale_table', 2)
+        per_stage = _run_dense(dev, a_q, a_s, b_q, b_s, variant=variant)
+    finally:
+        _lib.force_splitk(0)
+        _lib.tune('scale_table', 0)
+    helpers.tolerance_check(with_table, ref, f'scale table {variant}/{splitk} {M}x{N}x{K}')
+    assert torch.equal(with_table, per_stage)
+
+
+def test_refused_launch_enqueues_nothing(dev):
+    """A call whose main kernel cannot be launched (here: a forced request for more LDS than the GPU has) returns
+    DLB_ERR_LAUNCH before any pre-pass is enqueued: workspace and output keep their bytes."""
+    import ctypes
+    from dlblas_amd import _lib
+    lib = _lib.load()
+    M, N, K = 2048, 4096, 512  # row-major scales, 256-row tiles: the call starts with a scale re-layout pass
+    a_q, a_s, b_q, b_s = (t.to(dev) for t in helpers.make_dense(M, N, K, seed=5))
+    out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=dev)
+    ws = torch.full((_lib.WORKSPACE_BYTES, ), 0x5a, dtype=torch.uint8, device=dev)
+    ws[:_lib.WS_COUNTER_BYTES] = 0
+    vp = ctypes.c_void_p
+    args = (vp(a_q.data_ptr()), vp(b_q.data_ptr()), vp(a_s.data_ptr()), vp(b_s.data_ptr()), vp(out.data_ptr()), M, N, K, a_s.stride(0),
+            a_s.stride(1), _lib.OUT_BF16, vp(ws.data_ptr()), ws.numel(), vp(torch.cuda.current_stream().cuda_stream))
+    try:
+        _lib.tune('lds_oversize', 1)
+        rc = lib.dlb_fp8_gemm(*args)
+    finally:
+        _lib.tune('lds_oversize', 0)
+    torch.cuda.synchronize()
+    assert rc == _lib.ERR_LAUNCH and 'nothing enqueued' in _lib.last_error()
+    assert bool((ws[_lib.WS_COUNTER_BYTES:] == 0x5a).all()) and bool((out == 7.0).all())
+    assert lib.dlb_fp8_gemm(*args) == 0  # the same call goes through once the hook is off ...
+    torch.cuda.synchronize()
+    assert not bool((ws[_lib.WS_COUNTER_BYTES:] == 0x5a).all())  # ... and it does use the workspace
+    helpers.tolerance_check(out, orc.dequant_ref(a_q.cpu(), a_s.cpu(), b_q.cpu(), b_s.cpu()), 'after a refused launch')
+
+
 @pytest.mark.parametrize('variant', ['pipe256x256', 'pipe128x256w8', 'pipe256mix', 'pipe128x128', 'pipe128x64'])
 @pytest.mark.parametrize('M,N,K', [(200, 392, 2048), (513, 1032, 256)])
 def test_epilogue_through_lds_equals_direct_stores(dev, variant, M, N, K):

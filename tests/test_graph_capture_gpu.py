@@ -33,8 +33,17 @@ def test_decode_and_masked_gemm_replay_from_a_graph():
     static = {k: v.to(dev) for k, v in inputs[0].items()}
     gout = torch.full((G, M_max, GN), -7.0, dtype=torch.bfloat16, device=dev)
 
+    import ctypes
+    from dlblas_amd import _lib
+    lib, vp = _lib.load(), ctypes.c_void_p
+    na_out = torch.full((M, N), -3.0, dtype=torch.bfloat16, device=dev)
+
     def step():
         c = fp8_gemm(static['a_q'], static['b_q'], static['a_s'], static['b_s'])
+        # the entry point that works in the library's static scratch (bound to this stream by prepare())
+        _lib.check(lib.dlb_fp8_gemm_noalloc(vp(static['a_q'].data_ptr()), vp(static['b_q'].data_ptr()), vp(static['a_s'].data_ptr()),
+                                            vp(static['b_s'].data_ptr()), vp(na_out.data_ptr()), M, N, K, static['a_s'].stride(0),
+                                            static['a_s'].stride(1), _lib.OUT_BF16, vp(torch.cuda.current_stream().cuda_stream)))
         m_grouped_fp8_gemm_nt_masked((static['x_q'], static['x_s']), (static['w_q'], static['w_s']), gout,
                                      static['masked_m'], M_max // 2)
         return c
@@ -56,11 +65,14 @@ def test_decode_and_masked_gemm_replay_from_a_graph():
             torch.cuda.synchronize()
             graph.replay()
             torch.cuda.synchronize()
-            got_c, got_g = captured_c.clone(), gout.clone()
+            got_c, got_g, got_na = captured_c.clone(), gout.clone(), na_out.clone()
             gout.fill_(-7.0)
-            eager_c = step()
+            na_out.fill_(-3.0)
+            with torch.cuda.stream(side):
+                eager_c = step()
             torch.cuda.synchronize()
             assert torch.equal(got_c, eager_c) and torch.equal(got_g, gout), f'replay {rep} differs from the eager call'
+            assert torch.equal(got_na, eager_c) and torch.equal(na_out, eager_c), f'replay {rep}: the no-allocation entry point differs'
             helpers.tolerance_check(got_c, orc.dequant_ref(data['a_q'], data['a_s'], data['b_q'], data['b_s']), f'graph dense replay {rep}')
             ref = orc.grouped_masked_ref(data['x_q'], data['x_s'], data['w_q'], data['w_s'],
                                          torch.full((G, M_max, GN), -7.0, dtype=torch.float32), data['masked_m'])
