@@ -172,7 +172,8 @@ def time_steps(launch, steps, warmup):
     for _ in range(warmup):
         launch()
     wall, ev = _timed(launch, steps)
-    return wall, ev, {'ms_per_step': idle_wall, 'kernel_ms': idle_ev, 'settle_launches': settled}
+    return wall, ev, {'ms_per_step': idle_wall, 'kernel_ms': idle_ev, 'settle_launches': settled,
+                      'launches_before_the_timed_region': warmup + steps + settled + warmup}
 
 
 def cpu_baseline(kind, M, N, K, a_q, a_s, b_q, b_s, budget_s=12.0):
@@ -361,7 +362,21 @@ def ceilings(dev):
             ms = time_call(run, 20, 20)
             res['panel_stream_GBps'][f'{depth} K steps in flight, plus a shared (L2-resident) 256-row panel per step{tag}: HBM panel bytes only'] = \
                 panels * 256 * row_bytes / ms / 1e6
-    res['note'] = ('mfma_loop: pairs of v_mfma_f32_32x32x64_f8f6f4 + 16 scale FMAs from registers, 8 waves per CU, no memory '
+    # what the path from the L2 into a CU delivers when every request hits: all workgroups pull the same 512 rows, 64 KB per
+    # K step (the bytes a 256 x 256 tile needs per step), through the LDS DMA and through 16-byte register loads
+    lib.floor_l2_stream.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    res['l2_stream'] = {}
+    strip = torch.randint(0, 255, (512 * 18432, ), dtype=torch.uint8, device=dev)
+    steps_per_launch = 2000
+    for mode, name in ((0, 'LDS DMA'), (1, 'register loads')):
+        for depth in (1, 2):
+            def run(mode=mode, depth=depth):
+                lib.floor_l2_stream(ctypes.c_void_p(strip.data_ptr()), 18432, cus, steps_per_launch, mode, depth, stream)
+            ms = time_call(run, 10, 10)
+            res['l2_stream'][f'{name}, {depth} K steps in flight'] = {'GBps_per_cu': steps_per_launch * 65536 / ms / 1e6,
+                                                                       'ns_per_64KB_step': ms * 1e6 / steps_per_launch}
+    res['note'] = ('l2_stream: one workgroup per CU, every request an L2 hit after the first touch (the prefill kernel moves 64 KB '
+                   'per K step of about 1600 ns). mfma_loop: pairs of v_mfma_f32_32x32x64_f8f6f4 + 16 scale FMAs from registers, 8 waves per CU, no memory '
                    'traffic except the optional LDS reads (the prefill kernel issues 3 per pair); peak 5000 TFLOP/s. '
                    'panel_stream: one workgroup per CU pulls 256 x 7168-byte panels from HBM through the LDS DMA path, '
                    '128 bytes per row and K step, and computes nothing')
@@ -659,7 +674,7 @@ def fused_moe_workload(dev):
 
 def measured_traffic(workload):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 --pmc runs kept under profiles/ (None when
-    no counter run for this workload has been recorded)."""
+    no counter run for this workload has been recorded).  Not measured in this run: counters need the profiler."""
     path = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
     try:
         with open(path) as fh:
@@ -773,11 +788,14 @@ def main():
                     'unit': 'TFLOP/s'}
     roofline['frac'] = roofline['achieved'] / roofline['peak']
     roofline['traffic'] = measured_traffic(args.workload)
+    roofline['traffic_source'] = ('profiles/hbm_traffic.json: FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc runs of this command, '
+                                  'scaled by a 1 GiB copy; read from the committed file, not measured in this run')
     roofline['kernel_ms'] = ev_ms
     from_idle['frac_of_peak'] = (nbytes / 1e9 if memory_bound else flops / 1e12) / (from_idle['kernel_ms'] * 1e-3) / roofline['peak']
     from_idle['note'] = ('the same warmup + steps measured first, on an idle GPU: the power controller boosts, throttles and '
                          'recovers during the first tens of milliseconds of this load; value / roofline are measured after '
-                         'settle_launches further untimed launches, when the per-launch time has stopped moving')
+                         'settle_launches further untimed launches + one more warmup (effective_warmup_launches in all), when '
+                         'the per-launch time has stopped moving')
 
     result = {
         'metric': 'FP8 block-scaled GEMM TFLOP/s (% FP8 MFMA peak); decode-M HBM GB/s',
@@ -786,6 +804,9 @@ def main():
         'n_gpus': 1,
         'steps': args.steps,
         'warmup': args.warmup,
+        'effective_warmup_launches': from_idle['launches_before_the_timed_region'],
+        'from_idle_ms_per_step': from_idle['ms_per_step'],
+        'from_idle_frac_of_peak': from_idle['frac_of_peak'],
         'ms_per_step': ms_per_step,
         'higher_is_better': True,
         'scaling': 'weak',

@@ -11,6 +11,10 @@
 //   floor_panel_stream  one workgroup per CU streams 256-row panels of a row-major byte matrix through the LDS DMA path
 //                (global_load_lds_dwordx4, 8 rows x 128 bytes per wave instruction, K step by K step, S steps in
 //                flight) and does nothing with them: the rate at which a CU can pull a weight tile's rows from HBM
+//   floor_l2_stream  one workgroup per CU pulls the SAME 512 rows of a row-major byte matrix, 128 bytes per row and K
+//                step (the 64 KB a 256 x 256 GEMM tile needs per K step), so that after the first touch every request
+//                hits the L2: what the path from the L2 into a CU delivers, through the LDS DMA (S steps in flight) or
+//                through 16-byte register loads
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -120,7 +124,64 @@ __global__ void __launch_bounds__(512) floor_panel_stream_kernel(const char* src
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// MODE 0: global_load_lds_dwordx4 into a ring of S stages of 64 KB; MODE 1: global_load_dwordx4 into registers, the
+// loads of S K steps (8 per wave and step) in flight.  Workgroup b starts its walk over K at step 7 b (mod ksteps).
+template <int MODE, int S>
+__global__ void __launch_bounds__(512) floor_l2_stream_kernel(const char* src, int64_t row_bytes, int iters, int* sink) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ksteps = static_cast<int>(row_bytes / 128);
+  const char* base = src + (static_cast<int64_t>(wave) * 64 + (lane >> 3)) * row_bytes + (lane & 7) * 16;
+  int k = static_cast<int>((blockIdx.x * 7u) % static_cast<unsigned>(ksteps));
+  v4i acc = {0, 0, 0, 0};
+  for (int it = 0; it < iters; ++it) {
+    if (MODE == 0) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(base + static_cast<int64_t>(u) * 8 * row_bytes + k * 128),
+                                         (lds_ptr_t)(lds + ((it % S) * 64 + wave * 8 + u) * 1024), 16, 0, 0);
+      if (S == 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (S == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    } else {
+      v4i v[S][8];
+#pragma unroll
+      for (int s2 = 0; s2 < S; ++s2) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          v[s2][u] = *reinterpret_cast<const v4i*>(base + static_cast<int64_t>(u) * 8 * row_bytes + k * 128);
+        k = k + 1 == ksteps ? 0 : k + 1;
+      }
+#pragma unroll
+      for (int s2 = 0; s2 < S; ++s2)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[s2][u];
+      it += S - 1;
+      continue;
+    }
+    k = k + 1 == ksteps ? 0 : k + 1;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5a5a5a5a && sink == reinterpret_cast<int*>(1)) *sink = acc.x;
+}
+
 extern "C" {
+
+// src: [512][row_bytes] bytes; K steps of 64 KB per workgroup = iters; mode 0 = LDS DMA, 1 = register loads; depth = K
+// steps in flight (1 or 2)
+int floor_l2_stream(const void* src, int64_t row_bytes, int workgroups, int iters, int mode, int depth, void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const char* p = static_cast<const char*>(src);
+  if (row_bytes <= 0 || row_bytes % 128 != 0) return -1;
+  auto launch = [&](auto kernel, int lds_bytes) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) return;
+    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), lds_bytes, st, p, row_bytes, iters, nullptr);
+  };
+  if (mode == 0 && depth >= 2) launch(floor_l2_stream_kernel<0, 2>, 131072);
+  if (mode == 0 && depth < 2) launch(floor_l2_stream_kernel<0, 1>, 65536);
+  if (mode != 0 && depth >= 2) launch(floor_l2_stream_kernel<1, 2>, 0);
+  if (mode != 0 && depth < 2) launch(floor_l2_stream_kernel<1, 1>, 0);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
 
 int floor_empty(int workgroups, void* stream) {
   hipLaunchKernelGGL(floor_empty_kernel, dim3(workgroups), dim3(512), 0, static_cast<hipStream_t>(stream), nullptr);

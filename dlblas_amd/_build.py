@@ -23,17 +23,24 @@ def find_hipcc() -> str:
     raise RuntimeError('hipcc not found (set HIPCC or put /opt/rocm/bin on PATH)')
 
 
-def build_library(verbose: bool = False) -> str:
-    """Compile csrc/*.hip into libdlblas_fp8_gemm.so; always recompiles. Returns the library path."""
-    cmd = [find_hipcc()] + HIPCC_FLAGS + ['-o', LIB_PATH] + [os.path.join(CSRC_DIR, s) for s in SOURCES]
+def build_library(verbose: bool = False, defines=(), out_path: str = LIB_PATH) -> str:
+    """Compile csrc/*.hip into libdlblas_fp8_gemm.so; always recompiles. Returns the library path.
+    `defines` / `out_path`: measurement builds kept apart from the library (the DLB_ABLATE_* switches of the ring kernels'
+    K step, loaded through the DLBLAS_AMD_LIB environment variable)."""
+    cmd = [find_hipcc()] + HIPCC_FLAGS + [f'-D{d}' for d in defines] + ['-o', out_path] + [os.path.join(CSRC_DIR, s) for s in SOURCES]
     res = subprocess.run(cmd, cwd=CSRC_DIR, capture_output=True, text=True)
     log = '\n'.join(line for line in (res.stdout + res.stderr).splitlines() if 'packed-fp32-ops' not in line)
     if res.returncode != 0:
         raise RuntimeError(f'hipcc failed ({res.returncode}):\n{log}')
     if verbose and log.strip():
         print(log)
-    return LIB_PATH
+    return out_path
 
 
 if __name__ == '__main__':
-    print(build_library(verbose=True))
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--define', action='append', default=[], help='preprocessor symbol of a measurement build, e.g. DLB_ABLATE_VMCNT')
+    ap.add_argument('--out', default=LIB_PATH, help='output path (default: the library next to this file)')
+    a = ap.parse_args()
+    print(build_library(verbose=True, defines=a.define, out_path=a.out))

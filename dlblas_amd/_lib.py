@@ -12,7 +12,7 @@ import torch
 
 from ._build import LIB_PATH
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 OUT_BF16, OUT_F32 = 0, 1
 WS_COUNTER_BYTES = 65536
 WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
@@ -43,6 +43,7 @@ SYMBOLS = {
     'dlb_fp8_gemm_grouped_masked':
     (ctypes.c_int, [_c_vp] * 6 + [_c_i32] + [_c_i64] * 3 + [_c_i32] + [_c_i64] * 3 + [ctypes.c_int, _c_vp, _c_sz, _c_vp]),
     'dlb_fp8_quant_1x128': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
+    'dlb_fp8_quant_group': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 6 + [ctypes.c_float, _c_vp]),
     'dlb_fp8_quant_128x128': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 4 + [ctypes.c_float, _c_vp]),
     'dlb_fp8_gemm_force_variant': (ctypes.c_int, [ctypes.c_int]),
     'dlb_fp8_gemm_tune': (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
@@ -311,14 +312,18 @@ def gemm_masked_silu_quant(a, b, a_s, b_s, out_q, out_s, masked_m, expected_m, M
 IN_CODES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
 
-def quant_1x128(x2d, q, s, rows, K, x_row_stride, s_stride_m, s_stride_k, eps):
+def quant_group(x2d, q, s, rows, K, group_size, x_row_stride, s_stride_m, s_stride_k, eps):
     _require_gpu(x2d, q, s)
     lib = load()
     with torch.cuda.device(x2d.device):
         stream = torch.cuda.current_stream(x2d.device).cuda_stream
         check(
-            lib.dlb_fp8_quant_1x128(_ptr(x2d), IN_CODES[x2d.dtype], _ptr(q), _ptr(s), rows, K, x_row_stride, s_stride_m,
+            lib.dlb_fp8_quant_group(_ptr(x2d), IN_CODES[x2d.dtype], _ptr(q), _ptr(s), rows, K, group_size, x_row_stride, s_stride_m,
                                     s_stride_k, float(eps), ctypes.c_void_p(stream)))
+
+
+def quant_1x128(x2d, q, s, rows, K, x_row_stride, s_stride_m, s_stride_k, eps):
+    quant_group(x2d, q, s, rows, K, 128, x_row_stride, s_stride_m, s_stride_k, eps)
 
 
 def _stream(t: torch.Tensor):

@@ -949,6 +949,21 @@ int static_scratch_slice(hipStream_t stream, void** out) {
               "for this stream", DLB_STATIC_SCRATCH_SLICES, dev);
 }
 
+template <int IN>
+void launch_quant_group(const QuantArgs& qa, int lanes, unsigned blocks, hipStream_t st) {
+  const dim3 grid(blocks), block(256);
+  switch (lanes) {
+    case 1: hipLaunchKernelGGL((fp8_quant_group_kernel<IN, 1>), grid, block, 0, st, qa); break;
+    case 2: hipLaunchKernelGGL((fp8_quant_group_kernel<IN, 2>), grid, block, 0, st, qa); break;
+    case 4: hipLaunchKernelGGL((fp8_quant_group_kernel<IN, 4>), grid, block, 0, st, qa); break;
+    case 8: hipLaunchKernelGGL((fp8_quant_group_kernel<IN, 8>), grid, block, 0, st, qa); break;
+    case 16: hipLaunchKernelGGL((fp8_quant_group_kernel<IN, 16>), grid, block, 0, st, qa); break;
+    case 32: hipLaunchKernelGGL((fp8_quant_group_kernel<IN, 32>), grid, block, 0, st, qa); break;
+    case 64: hipLaunchKernelGGL((fp8_quant_group_kernel<IN, 64>), grid, block, 0, st, qa); break;
+    default: hipLaunchKernelGGL(fp8_quant_group_generic_kernel<IN>, grid, block, 0, st, qa);
+  }
+}
+
 }  // namespace
 }  // namespace dlb
 
@@ -1081,38 +1096,52 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
   return dlb::run(pr);
 }
 
-int dlb_fp8_quant_1x128(const void* x, int x_dtype, void* q, float* s, int64_t rows, int64_t K, int64_t x_row_stride,
-                        int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream) {
+int dlb_fp8_quant_group(const void* x, int x_dtype, void* q, float* s, int64_t rows, int64_t K, int64_t group_size,
+                        int64_t x_row_stride, int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream) {
   using namespace dlb;
   g_err[0] = '\0';
   if (x_dtype < kInBf16 || x_dtype > kInF32) return fail(DLB_ERR_BAD_DTYPE, "x_dtype %d is not DLB_IN_BF16 / F16 / F32", x_dtype);
   if (rows < 0 || K < 0) return fail(DLB_ERR_BAD_SHAPE, "negative dimension (rows=%lld K=%lld)", (long long)rows, (long long)K);
-  if (K % kScaleBlock != 0) return fail(DLB_ERR_BAD_SHAPE, "K=%lld is not a multiple of the group size 128", (long long)K);
+  if (group_size <= 0) return fail(DLB_ERR_BAD_SHAPE, "group size %lld is not positive", (long long)group_size);
+  if (K % group_size != 0)
+    return fail(DLB_ERR_BAD_SHAPE, "K=%lld is not a multiple of the group size %lld", (long long)K, (long long)group_size);
   if (rows == 0 || K == 0) return DLB_OK;
   if (!x || !q || !s) return fail(DLB_ERR_NULL_POINTER, "x, q or s is NULL");
   const int64_t esz = x_dtype == kInF32 ? 4 : 2;
   if (x_row_stride < K) return fail(DLB_ERR_BAD_STRIDE, "x row stride %lld < K", (long long)x_row_stride);
   if (s_stride_m < 0 || s_stride_k < 0) return fail(DLB_ERR_BAD_STRIDE, "negative scale stride");
-  if (misaligned(x, 16) || (x_row_stride * esz) % 16 != 0 || misaligned(q, 8) || misaligned(s, 4))
-    return fail(DLB_ERR_ALIGNMENT, "x rows must be 16-byte aligned, q 8-byte aligned");
+  if (misaligned(x, esz) || misaligned(s, 4)) return fail(DLB_ERR_ALIGNMENT, "x or s is not aligned to its element size");
+  // the vector kernel: whole 16-byte loads and 8-byte stores per lane
+  const bool vector_ok = group_size % 8 == 0 && group_size <= 512 && !misaligned(x, 16) && (x_row_stride * esz) % 16 == 0 && !misaligned(q, 8);
+  if (group_size == kScaleBlock && !vector_ok) return fail(DLB_ERR_ALIGNMENT, "x rows must be 16-byte aligned, q 8-byte aligned");
+  int lanes = 0;  // 0 = generic kernel
+  if (vector_ok)
+    for (lanes = 1; lanes * 8 < group_size; lanes *= 2) {
+    }
   int dev = 0;
   const int cus = device_cu_count(&dev);
   if (cus < 0) return fail(DLB_ERR_LAUNCH, "hipGetDevice failed");
-  QuantArgs qa{x, static_cast<uint8_t*>(q), s, rows, K / kScaleBlock, x_row_stride, s_stride_m, s_stride_k, eps};
-  const int64_t groups = rows * (K / kScaleBlock);
-  int64_t blocks = ceil_div(groups, 16);  // 4 waves x 4 groups per step
+  QuantArgs qa{x, static_cast<uint8_t*>(q), s, rows, K / group_size, group_size, x_row_stride, s_stride_m, s_stride_k, eps};
+  const int64_t groups = rows * (K / group_size);
+  const int64_t per_block = lanes > 0 ? 4 * (64 / lanes) : 4;  // 4 waves x groups per wave and step
+  int64_t blocks = ceil_div(groups, per_block);
   const int64_t cap = static_cast<int64_t>(cus) * 16;
   if (blocks > cap) blocks = cap;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (x_dtype == kInBf16)
-    hipLaunchKernelGGL(fp8_quant_1x128_kernel<kInBf16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, qa);
+    launch_quant_group<kInBf16>(qa, lanes, static_cast<unsigned>(blocks), st);
   else if (x_dtype == kInF16)
-    hipLaunchKernelGGL(fp8_quant_1x128_kernel<kInF16>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, qa);
+    launch_quant_group<kInF16>(qa, lanes, static_cast<unsigned>(blocks), st);
   else
-    hipLaunchKernelGGL(fp8_quant_1x128_kernel<kInF32>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, qa);
+    launch_quant_group<kInF32>(qa, lanes, static_cast<unsigned>(blocks), st);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(DLB_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
   return DLB_OK;
+}
+
+int dlb_fp8_quant_1x128(const void* x, int x_dtype, void* q, float* s, int64_t rows, int64_t K, int64_t x_row_stride,
+                        int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream) {
+  return dlb_fp8_quant_group(x, x_dtype, q, s, rows, K, dlb::kScaleBlock, x_row_stride, s_stride_m, s_stride_k, eps, stream);
 }
 
 int dlb_fp8_quant_128x128(const void* w, int w_dtype, void* q, float* s, int64_t G, int64_t N, int64_t K,

@@ -366,6 +366,9 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       constexpr int i = decltype(idx)::value;
       uint8_t* sbase = smem + stage * Cfg::STAGE_BYTES;
       if constexpr (i < Cfg::A_INST) {
+#ifdef DLB_ABLATE_A
+        return;
+#endif
         uint32_t o = a_off[i];
         asm volatile("" : "+v"(o));
         dma_16(a_tile + static_cast<int64_t>(kb) * kScaleBlock, o, sbase + (i * WAVES + wave) * 1024);
@@ -583,9 +586,18 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         const int si = t / H, hi = t % H;
         if (si == S - 1 && hi == 0) {
           // every LDS read of this stage has been issued and the barrier waits for their return: hand it over
+          // (DLB_ABLATE_*: measurement builds with one part of the K step compiled out - their results are wrong on
+          // purpose; what a launch gains by it is what that part costs.  Never defined in the library build.)
+#ifndef DLB_ABLATE_VMCNT
           wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
+#endif
+#ifndef DLB_ABLATE_BARRIER
           lds_barrier();
+#else
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#endif
         }
+#ifndef DLB_ABLATE_DMA
         if (t >= kP) {
           if (t - kP < kSlots) {
             if (t - kP == 0) issue_slot(std::integral_constant<int, 0>{}, kb_new, stage);
@@ -600,6 +612,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
           if (t + T - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_prev, prev_stage);
           if (t + T - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_prev, prev_stage);
         }
+#endif
         // The scheduling fences pin the order MFMA pair -> reloads -> scale FMAs; without them the compiler
         // hoists the reloads above the MFMAs into fresh registers and the kernel spills.
         __builtin_amdgcn_sched_barrier(0);
@@ -607,6 +620,16 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
 #pragma unroll
         for (int u = 0; u < 16; ++u) z[u] = 0.f;
         constexpr int kSlot = Cfg::PARTS == 2 ? 1 : 0;
+#ifdef DLB_ABLATE_MFMADEP
+        if (kHoldX) {  // the two MFMAs of a tile independent of each other (the first one's product is dropped)
+          v16f z2;
+#pragma unroll
+          for (int u = 0; u < 16; ++u) z2[u] = 0.f;
+          z = mfma_32x32x64_e4m3(sf[0], hf[hi][0], z);
+          part[t & kSlot] = mfma_32x32x64_e4m3(sf[1], hf[hi][1], z2);
+          asm volatile("" ::"v"(z));
+        } else
+#endif
         if (kHoldX) {
           z = mfma_32x32x64_e4m3(sf[0], hf[hi][0], z);
           part[t & kSlot] = mfma_32x32x64_e4m3(sf[1], hf[hi][1], z);
@@ -616,20 +639,35 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         }
         __builtin_amdgcn_sched_barrier(0);
         // in-place reloads: the MFMAs above were the last readers of these registers
+#ifndef DLB_ABLATE_LDSREAD
         if (hi == H - 1 && si + 1 < S) {
           sf[0] = lds_read_frag32(smem, cur_base + strm0 + (si + 1) * kFragBytes, lc, 0);
           sf[1] = lds_read_frag32(smem, cur_base + strm0 + (si + 1) * kFragBytes, lc, 1);
         }
         if (si == S - 1) {
+#ifndef DLB_ABLATE_A
           hf[hi][0] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 0);
           hf[hi][1] = lds_read_frag32(smem, nxt_base + held0 + hi * kFragBytes, lc, 1);
+#else
+          asm volatile("" : "+v"(hf[hi][0]), "+v"(hf[hi][1]));
+#endif
           if (hi == 0) load_scales(nxt_base, min(kb + 1, nk - 1), sc_next);
           if (hi == H - 1) {
             sf[0] = lds_read_frag32(smem, nxt_base + strm0, lc, 0);
             sf[1] = lds_read_frag32(smem, nxt_base + strm0, lc, 1);
           }
         }
+#else
+        if (si == S - 1 && hi == 0) load_scales(nxt_base, min(kb + 1, nk - 1), sc_next);
+        asm volatile("" : "+v"(sf[0]), "+v"(sf[1]), "+v"(hf[hi][0]), "+v"(hf[hi][1]));  // the operands change for all the compiler knows
+#endif
         __builtin_amdgcn_sched_barrier(0);
+#ifdef DLB_ABLATE_SCALE
+        {  // one of the 16 scale FMAs of a tile, so that its MFMAs stay
+          const int mi = kHoldX ? hi : si, ni = kHoldX ? si : hi;
+          acc[mi][ni][0] += part[t & kSlot][0] * sc[mi][kUniformW ? 0 : ni];
+        }
+#else
         if (Cfg::PARTS == 1) {
           // scale-and-accumulate this tile; the other wave of the SIMD owns the matrix pipe meanwhile
           const int mi = kHoldX ? hi : si, ni = kHoldX ? si : hi;
@@ -642,6 +680,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
           const int pmi = kHoldX ? pt % H : pt / H, pni = kHoldX ? pt / H : pt % H;
           acc[pmi][pni] += part[pt & 1] * sc[pmi][kUniformW ? 0 : pni];
         }
+#endif
       }
       sc_last = sc[MF - 1][NS - 1];
 #pragma unroll

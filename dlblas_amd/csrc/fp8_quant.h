@@ -1,8 +1,11 @@
-// 1 x 128 activation quantiser for gfx950: per row and 128-wide group, s = max(amax, eps) / 448 and
-// q = clamp(x / s, -448, 448) rounded to nearest-even e4m3fn.  Restates _per_token_group_quant_fp8 and its
-// column-major-scale twin (dlblas/kernels/fp8.py:8-105).  HBM-bound: every element is read once (16-byte loads,
-// 8 elements per lane) and written once (8-byte stores); 16 lanes share a group and reduce its amax with DPP-style
-// shuffles, so a wave handles 4 groups per step.
+// Per-token-group activation quantiser for gfx950: per row and group of `group_size` consecutive elements,
+// s = max(amax, eps) / 448 and q = clamp(x / s, -448, 448) rounded to nearest-even e4m3fn.  Restates
+// _per_token_group_quant_fp8 and its column-major-scale twin (dlblas/kernels/fp8.py:8-105), whose group size is any
+// divisor of the row length (:35-36, BLOCK = next_power_of_2(group_size), lanes past the group masked).  HBM-bound:
+// every element is read once (16-byte loads, 8 elements per lane) and written once (8-byte stores); LANES lanes
+// (the power of two at or above group_size / 8) share a group and reduce its amax with DPP-style shuffles, so a wave
+// handles 64 / LANES groups per step: 16 lanes and 4 groups for the 128-wide groups of the block-scaled GEMM.  Group
+// sizes that are no multiple of 8, or beyond 512, take fp8_quant_group_generic_kernel (a wave per group, element loads).
 #pragma once
 
 #include "fp8_gemm_common.h"
@@ -14,7 +17,8 @@ struct QuantArgs {
   uint8_t* q;
   float* s;
   int64_t rows;
-  int64_t groups_per_row;  // K / 128
+  int64_t groups_per_row;  // K / group_size
+  int64_t group_size;
   int64_t x_row_stride;    // elements
   int64_t s_stride_m;      // floats
   int64_t s_stride_k;
@@ -77,28 +81,35 @@ __device__ __forceinline__ void quant_load8(const void* x, int64_t elem, float (
 // ALU-bound.
 __device__ __forceinline__ float div_by_scale(float v, float s, float r) { return act_div_by_scale(v, s, r); }
 
-template <int IN>
-__global__ void __launch_bounds__(256) fp8_quant_1x128_kernel(const QuantArgs p) {
+template <int IN, int LANES>
+__global__ void __launch_bounds__(256) fp8_quant_group_kernel(const QuantArgs p) {
+  constexpr int kPerWave = 64 / LANES;  // groups per wave and step
   const int lane = threadIdx.x & 63;
-  const int sub = lane & 15;  // position inside the group: elements 8 sub .. 8 sub + 7
+  const int sub = lane & (LANES - 1);  // position inside the group: elements 8 sub .. 8 sub + 7
   const int64_t total = p.rows * p.groups_per_row;
   const int64_t wave_id = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) >> 6;
   const int64_t n_waves = (static_cast<int64_t>(gridDim.x) * 256) >> 6;
-  for (int64_t g0 = wave_id * 4; g0 < total; g0 += n_waves * 4) {
-    const int64_t g = g0 + (lane >> 4);
-    const bool live = g < total;
-    const int64_t gc = live ? g : total - 1;
+  const bool in_group = sub * 8 < p.group_size;  // lanes past a group that is no power of two take no part
+  for (int64_t g0 = wave_id * kPerWave; g0 < total; g0 += n_waves * kPerWave) {
+    const int64_t g = g0 + lane / LANES;
+    const bool live = g < total && in_group;
+    const int64_t gc = g < total ? g : total - 1;
     // 32-bit division where it fits: the 64-bit one costs more than the rest of the loop body
     const int64_t row = total < (1ll << 31) ? static_cast<int64_t>(static_cast<uint32_t>(gc) / static_cast<uint32_t>(p.groups_per_row))
                                             : gc / p.groups_per_row;
     const int64_t kg = gc - row * p.groups_per_row;
     float v[8];
-    quant_load8<IN>(p.x, row * p.x_row_stride + kg * 128 + sub * 8, v);
+    if (in_group) {
+      quant_load8<IN>(p.x, row * p.x_row_stride + kg * p.group_size + sub * 8, v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = 0.f;
+    }
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
 #pragma unroll
-    for (int off = 8; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 16));
+    for (int off = LANES / 2; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, LANES));
     const float scale = fmaxf(amax, p.eps) / 448.0f;
     const float inv_scale = 1.0f / scale;
     int packed[2];
@@ -112,9 +123,41 @@ __global__ void __launch_bounds__(256) fp8_quant_1x128_kernel(const QuantArgs p)
       packed[i] = w;
     }
     if (live) {
-      *reinterpret_cast<v2i*>(p.q + (row * p.groups_per_row + kg) * 128 + sub * 8) = v2i{packed[0], packed[1]};
+      *reinterpret_cast<v2i*>(p.q + (row * p.groups_per_row + kg) * p.group_size + sub * 8) = v2i{packed[0], packed[1]};
       if (sub == 0) p.s[row * p.s_stride_m + kg * p.s_stride_k] = scale;
     }
+  }
+}
+
+// Any group size: a wave per group, lane l takes elements l, l + 64, ... with element-sized loads and byte stores, the
+// same arithmetic (correctly rounded quotient, hardware e4m3 cast).  Slow next to the kernel above; it is the general
+// case of the reference's signature, not a path of the GEMM.
+template <int IN>
+__global__ void __launch_bounds__(256) fp8_quant_group_generic_kernel(const QuantArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t total = p.rows * p.groups_per_row;
+  const int64_t n_waves = (static_cast<int64_t>(gridDim.x) * 256) >> 6;
+  auto element = [&](int64_t idx) -> float {
+    if (IN == kInF32) return static_cast<const float*>(p.x)[idx];
+    const uint32_t w = static_cast<const uint16_t*>(p.x)[idx];
+    if (IN == kInBf16) return __uint_as_float(w << 16);
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w)));
+  };
+  for (int64_t g = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) >> 6; g < total; g += n_waves) {
+    const int64_t row = g / p.groups_per_row, kg = g - row * p.groups_per_row;
+    const int64_t x0 = row * p.x_row_stride + kg * p.group_size;
+    float amax = 0.f;
+    for (int64_t e = lane; e < p.group_size; e += 64) amax = fmaxf(amax, fabsf(element(x0 + e)));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    const float scale = fmaxf(amax, p.eps) / 448.0f;
+    const float inv_scale = 1.0f / scale;
+    uint8_t* q0 = p.q + g * p.group_size;
+    for (int64_t e = lane; e < p.group_size; e += 64) {
+      const float c = fminf(fmaxf(div_by_scale(element(x0 + e), scale, inv_scale), -448.0f), 448.0f);
+      q0[e] = static_cast<uint8_t>(__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xff);
+    }
+    if (lane == 0) p.s[row * p.s_stride_m + kg * p.s_stride_k] = scale;
   }
 }
 

@@ -2,7 +2,8 @@
 
 Drop-in for ``per_token_group_quant_fp8`` of the reference (dlblas/kernels/fp8.py:108-182): same signature, same
 assertions, same output shapes (including the column-major scale view), computed by a hand-written gfx950 kernel
-through the C ABI.  Only group_size 128 and float8_e4m3fn are implemented (the block-scaled GEMM takes nothing else).
+through the C ABI.  Any group size that divides the row length is taken, as in the reference (the block-scaled GEMM uses
+128); only float8_e4m3fn is implemented, which is also all the reference supports (:124-125).
 """
 from typing import Optional, Tuple
 
@@ -13,11 +14,12 @@ from ..utils import SymVar, Tensor, register_dlblas_op
 
 
 @torch.library.custom_op('dlblas::per_token_group_quant_fp8', mutates_args=('x_q', 'x_s'), device_types='cuda')
-def quant_op(x: torch.Tensor, x_q: torch.Tensor, x_s: torch.Tensor, eps: float) -> None:
+def quant_op(x: torch.Tensor, x_q: torch.Tensor, x_s: torch.Tensor, eps: float, group_size: int = 128) -> None:
     K = x.shape[-1]
     rows = x.numel() // K
     row_stride = x.stride(-2) if x.dim() >= 2 else K
-    _lib.quant_1x128(x, x_q, x_s, rows, K, row_stride, x_s.stride(-2) if x_s.dim() >= 2 else K // 128, x_s.stride(-1), eps)
+    _lib.quant_group(x, x_q, x_s, rows, K, group_size, row_stride, x_s.stride(-2) if x_s.dim() >= 2 else K // group_size,
+                     x_s.stride(-1), eps)
 
 
 def per_token_group_quant_fp8(
@@ -35,8 +37,6 @@ def per_token_group_quant_fp8(
     assert (x.shape[-1] % group_size == 0), (
         f"the last dimension of 'x' {x.shape[-1]} must be divisible by 'group_size' {group_size}")
     assert x.stride(-1) == 1, f'{x} groups must be contiguous'
-    if group_size != 128:
-        raise NotImplementedError(f'only group_size 128 is implemented, got {group_size}')
     if dtype != torch.float8_e4m3fn:
         raise NotImplementedError(f'only float8_e4m3fn is implemented, got {dtype}')
     if x.dtype not in _lib.IN_CODES:
@@ -57,7 +57,7 @@ def per_token_group_quant_fp8(
     else:
         x_s = torch.empty(x.shape[:-1] + (K // group_size, ), device=x.device, dtype=torch.float32)
         s2d = x_s.reshape(rows, K // group_size)
-    quant_op(x2d, x_q.reshape(-1, K), s2d, float(eps))
+    quant_op(x2d, x_q.reshape(-1, K), s2d, float(eps), int(group_size))
     return x_q, x_s
 
 

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define DLB_ABI_VERSION 5
+#define DLB_ABI_VERSION 6
 
 /* output element type of C */
 #define DLB_OUT_BF16 0
@@ -266,6 +266,17 @@ int dlb_fp8_gemm_grouped_masked_silu_quant(const void* a, const void* b, const f
  */
 int dlb_fp8_quant_1x128(const void* x, int x_dtype, void* q, float* s, int64_t rows, int64_t K, int64_t x_row_stride,
                         int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream);
+
+/*
+ * The same quantiser for any group size, as per_token_group_quant_fp8 takes it (dlblas/kernels/fp8.py:108-182:
+ * group_size is any divisor of the row length, BLOCK = next_power_of_2(group_size)):
+ *     s[m, j] = max(max |x[m, group_size j ..]|, eps) / 448,   q = round_to_nearest_even_e4m3(clamp(x / s, -448, 448))
+ * with s [rows, K / group_size] addressed through (s_stride_m, s_stride_k).  K % group_size == 0 is required.  Group
+ * sizes that are a multiple of 8 up to 512 on 16-byte aligned rows run at memory speed (dlb_fp8_quant_1x128 is this
+ * function at group_size 128); anything else takes a slower element-wise kernel with the same arithmetic.
+ */
+int dlb_fp8_quant_group(const void* x, int x_dtype, void* q, float* s, int64_t rows, int64_t K, int64_t group_size,
+                        int64_t x_row_stride, int64_t s_stride_m, int64_t s_stride_k, float eps, void* stream);
 
 /*
  * 128 x 128 block quantiser, the producer of (b, b_s): one scale per block of the weight matrix, blocks at the N and

@@ -7,7 +7,7 @@ Each function restates one piece of the reference (paths relative to the DLBlas 
   dequant_ref                    the closed form of the test's ``gt`` fixture, tests/kernels/test_fp8_gemm.py:33-68
                                  = the arithmetic of fp8_gemm_kernel, dlblas/kernels/fp8_gemm.py:49-60
   dequant_ref_blocked            the same fixture in its original block-looped shape (:57-65)
-  quant_act_1x128                per_token_group_quant_fp8, dlblas/kernels/fp8.py:44-51,108-182
+  quant_act_group / _1x128       per_token_group_quant_fp8 (any group size / 128), dlblas/kernels/fp8.py:44-51,108-182
   quant_weight_128x128           128 x 128 block quantiser; the reference has none in the package, the scheme
                                  (block amax / 448) is that of its test data builder,
                                  tests/kernels/test_fused_moe_v2.py:35-60
@@ -123,17 +123,23 @@ def dequant_ref_blocked(a_q, a_s, b_q, b_s, out_dtype=torch.float32) -> torch.Te
 # ---------------------------------------------------------------------------------------------------------------
 # quantisers
 # ---------------------------------------------------------------------------------------------------------------
-def quant_act_1x128(x: torch.Tensor, eps: float = 1e-10):
-    """Per row and 128-wide group: ``s = max(amax, eps) / 448``, ``q = clamp(x / s, -448, 448)`` cast RTNE to e4m3fn.
+def quant_act_group(x: torch.Tensor, group_size: int, eps: float = 1e-10):
+    """Per row and group of ``group_size`` consecutive elements (any divisor of K, dlblas/kernels/fp8.py:35-51):
+    ``s = max(amax, eps) / 448``, ``q = clamp(x / s, -448, 448)`` cast RTNE to e4m3fn.
 
-    x [..., K] with K % 128 == 0.  Returns (q e4m3fn [..., K], s f32 [..., K/128]).
+    x [..., K] with K % group_size == 0.  Returns (q e4m3fn [..., K], s f32 [..., K / group_size]).
     """
-    assert x.shape[-1] % BLOCK == 0
-    xf = x.float().reshape(*x.shape[:-1], x.shape[-1] // BLOCK, BLOCK)
+    assert x.shape[-1] % group_size == 0
+    xf = x.float().reshape(*x.shape[:-1], x.shape[-1] // group_size, group_size)
     amax = xf.abs().amax(dim=-1, keepdim=True).clamp_min(eps)
     s = amax / E4M3_MAX
     q = (xf / s).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
     return q.reshape(x.shape), s.squeeze(-1).contiguous()
+
+
+def quant_act_1x128(x: torch.Tensor, eps: float = 1e-10):
+    """quant_act_group at the group size of the block-scaled GEMM: (q e4m3fn [..., K], s f32 [..., K/128])."""
+    return quant_act_group(x, BLOCK, eps)
 
 
 def quant_weight_128x128(w: torch.Tensor, eps: float = 1e-10):

@@ -1,4 +1,5 @@
-"""GPU parity of the 1 x 128 activation quantiser against the CPU oracle: byte-exact codes, bit-exact scales."""
+"""GPU parity of the per-token-group activation quantiser (1 x 128 and any other group size) and of the 128 x 128 weight
+quantiser against the CPU oracle: byte-exact codes, bit-exact scales."""
 import pytest
 import torch
 
@@ -40,6 +41,29 @@ def test_quant_matches_oracle_bit_for_bit(dev, dtype, M, K):
     g = helpers.gen(31)
     x = (torch.randn(M, K, generator=g) * 3).to(dtype)
     _check(x, dev)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('group_size,M,K', [(32, 40, 256), (64, 300, 7168), (256, 33, 1024), (512, 20, 2048), (96, 50, 960), (8, 9, 64),
+                                             (1024, 6, 2048), (100, 17, 700), (1, 5, 24), (2048, 3, 2048)])
+def test_quant_any_group_size(dev, dtype, group_size, M, K):
+    """The reference's signature takes any group size that divides the row (dlblas/kernels/fp8.py:35-36,147): multiples
+    of 8 up to 512 run on the vector kernel (lanes past a group that is no power of two are masked), the rest on the
+    element-wise kernel.  Byte-exact codes, bit-exact scales, row-major and column-major scale layouts."""
+    from dlblas_amd.kernels.fp8 import per_token_group_quant_fp8
+    print(f'case quant group_size={group_size} {dtype} M={M} K={K}', flush=True)
+    g = helpers.gen(35)
+    x = (torch.randn(M, K, generator=g) * 2).to(dtype)
+    x[0, :group_size] = 0   # an all-zero group takes the eps scale
+    q_ref, s_ref = orc.quant_act_group(x, group_size)
+    for column_major in (False, True):
+        q, s = per_token_group_quant_fp8(x.to(dev), group_size, column_major_scales=column_major)
+        torch.cuda.synchronize()
+        assert tuple(s.shape) == (M, K // group_size) and torch.equal(s.cpu(), s_ref)
+        if column_major:
+            assert s.stride(0) == 1
+        got, want = q.cpu().view(torch.uint8), q_ref.view(torch.uint8)
+        assert bool(((got == want) | (((got | want) & 0x7F) == 0)).all()), f'{int((got != want).sum())} codes differ'
 
 
 def test_quant_edge_values(dev):

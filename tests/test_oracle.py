@@ -162,6 +162,33 @@ def test_act_quantiser_invariants():
     assert torch.all((recon - xf).abs() <= bound)
 
 
+@pytest.mark.parametrize('group_size', [1, 8, 32, 96, 100, 256, 600])
+def test_act_quantiser_any_group_size(group_size):
+    """quant_act_group with the group size the reference's signature allows (any divisor of the row length): the same
+    invariants per group, and at 128 it is quant_act_1x128."""
+    g = helpers.gen(6)
+    K = group_size * 6
+    x = (torch.randn(11, K, generator=g) * 5).to(torch.bfloat16)
+    x[2, group_size:2 * group_size] = 0
+    q, s = orc.quant_act_group(x, group_size)
+    assert s.shape == (11, 6)
+    qf, xf = orc.decode_e4m3fn(q).reshape(11, 6, group_size), x.float().reshape(11, 6, group_size)
+    amax = xf.abs().amax(-1)
+    assert torch.allclose(s, amax.clamp_min(1e-10) / 448, rtol=1e-6, atol=0)
+    assert (qf[2, 1] == 0).all() and s[2, 1] == pytest.approx(1e-10 / 448, rel=1e-5)
+    assert torch.all(qf.abs().amax(-1)[amax > 0] == 448)
+    bound = torch.maximum(xf.abs() * 2.0**-4, s[..., None] * 2.0**-10) * 1.0001
+    assert torch.all((qf * s[..., None] - xf).abs() <= bound)
+    # a group is quantised on its own: the same group as a matrix of one group gives the same codes and scale
+    q1, s1 = orc.quant_act_group(x[:, 3 * group_size:4 * group_size].contiguous(), group_size)
+    assert torch.equal(q1.view(torch.uint8), q[:, 3 * group_size:4 * group_size].view(torch.uint8)) and torch.equal(s1[:, 0], s[:, 3])
+    if group_size == 8:
+        x128 = (torch.randn(4, 256, generator=g)).to(torch.bfloat16)
+        qa, sa = orc.quant_act_group(x128, 128)
+        qb, sb = orc.quant_act_1x128(x128)
+        assert torch.equal(qa.view(torch.uint8), qb.view(torch.uint8)) and torch.equal(sa, sb)
+
+
 def test_weight_quantiser_blocks_and_ragged_edges():
     g = helpers.gen(6)
     w = (torch.randn(300, 200, generator=g) * 0.02).to(torch.bfloat16)
