@@ -192,7 +192,7 @@ def force_variant(name_or_id) -> None:
 
 
 KNOBS = {'splitk': 0, 'skinny_waves': 1, 'skinny_unroll': 2, 'skinny_nfrags': 3, 'group_m': 4, 'skinny_dma': 5, 'epilogue': 6, 'skinny_bn': 7,
-         'splitk_mode': 8, 'spin_limit': 9, 'scale_table': 10, 'lds_oversize': 11}
+         'splitk_mode': 8, 'spin_limit': 9, 'scale_table': 10, 'lds_oversize': 11, 'masked_grid': 12}
 
 
 def tune(knob: str, value) -> None:

@@ -97,9 +97,10 @@ enum Knob : int {
   kKnobSpinLimit,  // one-launch split-K: value - 1 polls for the other slices of a tile (0 = default; 1 = none: the last arrival adds every share)
   kKnobScaleTable, // 0 / 1: row-major activation scales of the small ring kernels go through the per-tile table, 2: never
   kKnobLdsOversize,  // test hook: 1 = ask for more LDS than the GPU has, so that the launch is refused before anything is enqueued
+  kKnobMaskedGrid,   // workgroups per CU of the masked layout's persistent grid (0 = default)
   kKnobCount
 };
-thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 // set while run() asks every kernel of the call for its launch attributes, before the first pre-pass is enqueued
 thread_local bool g_prepare_only = false;
 constexpr int kDefaultSpinLimit = 400;  // x about 0.5 us: far beyond the spread of the slices of one round of workgroups
@@ -141,7 +142,11 @@ constexpr int kListLds = Pipe256x256::LDS_BYTES > Pipe128x256w8::LDS_BYTES
                              ? (Pipe256x256::LDS_BYTES > Pipe192x256::LDS_BYTES ? Pipe256x256::LDS_BYTES : Pipe192x256::LDS_BYTES)
                              : (Pipe128x256w8::LDS_BYTES > Pipe192x256::LDS_BYTES ? Pipe128x256w8::LDS_BYTES : Pipe192x256::LDS_BYTES);
 // small tiles for problems with few of the large ones (M of a few hundred, or a narrow N): 4 waves, deep rings
+#ifdef DLB_EXP_P128
+typedef PipeCfg<2, 2, 2, 2, DLB_EXP_P128, 2, false> Pipe128x128;  // experiment: 4 waves, in-place K loop, DLB_EXP_P128 stages
+#else
 typedef PipeCfg<2, 2, 2, 2, 4, 2, true> Pipe128x128;  // wave tile 64 x 64, 4 stages of 34 KB
+#endif
 typedef PipeCfg<2, 2, 2, 1, 5, 2, true> Pipe128x64;   // wave tile 64 x 32, 5 stages of 26 KB
 // the same with the activation scales of a tile in a table behind the ring (row-major a_s, at most 32 K blocks per workgroup)
 typedef PipeCfg<2, 2, 2, 2, 4, 2, true, true> Pipe128x128T;
@@ -609,9 +614,12 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
   const int64_t tiles_m = ceil_div(rows, pl.bm), tiles_n = ceil_div(N, pl.bn);
   int64_t grid = tiles_m * tiles_n * r.splitk;
   if (mode == kMasked) {
-    // the real tile count is only known on the device; cover the worst case with a resident-sized grid
+    // the real tile count is only known on the device: a persistent grid
     const int64_t worst = tiles_m * tiles_n * G;
-    grid = worst < static_cast<int64_t>(cus) * 4 ? worst : static_cast<int64_t>(cus) * 4;
+    // One resident workgroup per CU that walks its tiles: equal tiles need no balancing by the hardware's dispatcher,
+    // and every further workgroup a CU has to start costs it about 2 us (32 x 256 x 7168 x 2048: 145 -> 137 us).
+    const int64_t per_cu = g_knob[kKnobMaskedGrid] > 0 ? g_knob[kKnobMaskedGrid] : 1;
+    grid = worst < static_cast<int64_t>(cus) * per_cu ? worst : static_cast<int64_t>(cus) * per_cu;
     grid = (grid + 31) / 32 * 32;  // the ring kernels deal tiles to the XCDs four at a time
   }
   // Dense launches of many rounds of equal tiles run one resident workgroup per CU that walks its tiles itself (the

@@ -430,12 +430,19 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
               (r * static_cast<uint32_t>(p.as_sm) + j * static_cast<uint32_t>(p.as_sk)) * 4u, smem + Cfg::SCTAB_OFF + i * 256);
       }
     }
+    // kExactK: only K blocks that exist are fetched - a tile shorter than the ring, and the last STAGES steps of every
+    // tile, issue nothing (wave-uniform branches), so no load is in flight when the tile ends and the next tile starts
+    // without waiting for loads nobody reads.  The kernels whose wave tile fills the register file (64 x 128) cannot
+    // afford those branches' scalar registers inside the K loop (wave tiles above 64 x 64): they keep every step the same code, fetch the last
+    // block again past the end of K into a stage nobody reads, and drain at the end of the tile.
+    constexpr bool kExactK = MF * NF <= 4;
 #pragma unroll
-    for (int s = 0; s < STAGES; ++s) issue_stage(min(s, nk - 1), s);
-    if (STAGES >= 3)
-      wait_vmcnt<(STAGES - 1) * Cfg::LOADS_PER_STAGE>();
+    for (int s = 0; s < STAGES; ++s)
+      if (!kExactK || s < nk) issue_stage(min(s, nk - 1), s);
+    if (!kExactK || nk >= STAGES)
+      wait_vmcnt<(STAGES - 1) * Cfg::LOADS_PER_STAGE>();  // all but the first stage's group may still be on their way
     else
-      wait_vmcnt<Cfg::LOADS_PER_STAGE>();
+      wait_vmcnt<0>();
     lds_barrier();
 
     if constexpr (Cfg::PREFETCH) {
@@ -477,17 +484,21 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         wr[0][ni][1] = lds_read_frag32(smem, w0 + ni * kFragBytes, lc, 1);
       }
 
-      // Every step is the same code: a step always hands its stage to the DMA (past the end of K the DMA re-reads
-      // the last block into a stage nobody reads) and always prefetches "the next stage" (garbage after the last
-      // one, never used), so exactly STAGES - 1 DMA groups are in flight at every barrier and nothing is peeled.
+      // Every step is the same code: a step always prefetches "the next stage" into registers (garbage after the
+      // last one, never used); whether it hands its stage to the DMA and how many groups it leaves in flight at its
+      // barrier are wave-uniform branches on the step's distance from the end of K.
       auto k_step = [&](auto buf_tag, int kb, int stage) __attribute__((always_inline)) {
         constexpr int B = decltype(buf_tag)::value;
         const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
         const int nxt_base = next_stage * Cfg::STAGE_BYTES;
         // every wave holds this stage's fragments in registers and has its share of the next stage in LDS
-        wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
+        // the group of step kb + 1 has landed: behind it at most STAGES - 2 younger groups are out, fewer at the tile's end
+        if (kExactK && kb + STAGES > nk)
+          wait_vmcnt<0>();
+        else
+          wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
         lds_barrier();
-        issue_stage(min(kb + STAGES, nk - 1), stage);
+        if (!kExactK || kb + STAGES < nk) issue_stage(min(kb + STAGES, nk - 1), stage);
 #pragma unroll
         for (int t = 0; t < T; ++t) {
           const int mi = t / NF, ni = t % NF;
@@ -527,7 +538,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       }
       if (kb < nk) k_step(B0{}, kb, stage);
       acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc_last;
-      wait_vmcnt<0>();  // the trailing re-read groups must not land in the next tile's ring
+      if (!kExactK) wait_vmcnt<0>();  // the trailing re-read groups must not land in the next tile's ring
     } else {
     v8i hf[H][2];
     v8i sf[2];
@@ -571,7 +582,8 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       constexpr int kSlots = T >= 8 ? 5 : (T >= 4 ? 3 : 1);  // measured: 3 to 5 of 8 slots are equally good, 6 and 7 leave the loads too little time
       constexpr int L = Cfg::LOADS_PER_STAGE;
       const int prev_stage = stage == 0 ? STAGES - 1 : stage - 1;
-      const int kb_new = min(kb + STAGES, nk - 1), kb_prev = min(kb + STAGES - 1, nk - 1);
+      const int kb_new = kExactK ? kb + STAGES : min(kb + STAGES, nk - 1), kb_prev = kExactK ? kb + STAGES - 1 : min(kb + STAGES - 1, nk - 1);
+      const bool do_new = !kExactK || kb_new < nk, do_prev = !kExactK || kb_prev < nk;  // kExactK: K blocks past the end are not fetched
       auto issue_slot = [&](auto qtag, int kbx, int stg) __attribute__((always_inline)) {
         constexpr int q = decltype(qtag)::value;
         constexpr int i0 = q * L / kSlots, i1 = (q + 1) * L / kSlots;
@@ -589,7 +601,11 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
           // (DLB_ABLATE_*: measurement builds with one part of the K step compiled out - their results are wrong on
           // purpose; what a launch gains by it is what that part costs.  Never defined in the library build.)
 #ifndef DLB_ABLATE_VMCNT
-          wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
+          // the group of step kb + 1 has landed: behind it at most STAGES - 2 younger groups are out, fewer at the tile's end
+          if (kExactK && kb + STAGES > nk)
+            wait_vmcnt<0>();
+          else
+            wait_vmcnt<(STAGES - 2) * Cfg::LOADS_PER_STAGE>();
 #endif
 #ifndef DLB_ABLATE_BARRIER
           lds_barrier();
@@ -599,14 +615,14 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         }
 #ifndef DLB_ABLATE_DMA
         if (t >= kP) {
-          if (t - kP < kSlots) {
+          if (t - kP < kSlots && do_new) {
             if (t - kP == 0) issue_slot(std::integral_constant<int, 0>{}, kb_new, stage);
             if (t - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_new, stage);
             if (t - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_new, stage);
             if (t - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_new, stage);
             if (t - kP == 4) issue_slot(std::integral_constant<int, 4>{}, kb_new, stage);
           }
-        } else if (t + T - kP < kSlots) {
+        } else if (t + T - kP < kSlots && do_prev) {
           if (t + T - kP == 1) issue_slot(std::integral_constant<int, 1>{}, kb_prev, prev_stage);
           if (t + T - kP == 2) issue_slot(std::integral_constant<int, 2>{}, kb_prev, prev_stage);
           if (t + T - kP == 3) issue_slot(std::integral_constant<int, 3>{}, kb_prev, prev_stage);
@@ -694,7 +710,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       stage = stage + 1 == STAGES ? 0 : stage + 1;
     }
     if (Cfg::PARTS == 2) acc[MF - 1][NF - 1] += part[(T - 1) & 1] * sc_last;
-    wait_vmcnt<0>();  // the trailing re-read groups must not land in the next tile's ring
+    if (!kExactK) wait_vmcnt<0>();  // the trailing re-read groups must not land in the next tile's ring
     }
 
     // epilogue: lane holds c[m0 + wm0 + 32 mi + (lane & 31)][n0 + wn0 + 32 ni + 8 u + 4 (lane >> 5) + 0..3], u = 0..3

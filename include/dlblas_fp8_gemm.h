@@ -334,6 +334,7 @@ int dlb_fp8_gemm_force_variant(int variant);
  *                           (1 = none: the workgroup that completes a tile adds all of it)
  *   DLB_KNOB_SCALE_TABLE    2 = the small DMA-ring kernels fetch row-major activation scales stage by stage instead of
  *                           once per tile into a table in LDS
+ *   DLB_KNOB_MASKED_GRID    workgroups per CU of the persistent grid of the masked layout (default 1)
  *   DLB_KNOB_LDS_OVERSIZE   test hook: 1 = every kernel asks for more LDS than the GPU has, so the call is refused
  *                           (DLB_ERR_LAUNCH) before anything is enqueued
  */
@@ -349,6 +350,7 @@ int dlb_fp8_gemm_force_variant(int variant);
 #define DLB_KNOB_SPIN_LIMIT 9
 #define DLB_KNOB_SCALE_TABLE 10
 #define DLB_KNOB_LDS_OVERSIZE 11
+#define DLB_KNOB_MASKED_GRID 12
 int dlb_fp8_gemm_tune(int knob, int value);
 
 /* Name of kernel variant `variant`, or NULL beyond the last one. */
