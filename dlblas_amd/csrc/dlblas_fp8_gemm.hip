@@ -151,6 +151,8 @@ typedef PipeCfg<2, 2, 2, 1, 5, 2, true> Pipe128x64;   // wave tile 64 x 32, 5 st
 // the same with the activation scales of a tile in a table behind the ring (row-major a_s, at most 32 K blocks per workgroup)
 typedef PipeCfg<2, 2, 2, 2, 4, 2, true, true> Pipe128x128T;
 typedef PipeCfg<2, 2, 2, 1, 5, 2, true, true> Pipe128x64T;
+typedef PipeCfg<2, 4, 2, 2, 3, 2, false, true, 16> Pipe128x256w8T;  // the masked layout's tiles (K of at most 16 blocks: 8 KB next to the 150 KB ring)
+static_assert(Pipe128x256w8T::LDS_BYTES <= 160 * 1024 && Pipe128x128T::LDS_BYTES <= 160 * 1024 && Pipe128x64T::LDS_BYTES <= 160 * 1024, "ring + table fit the LDS");
 constexpr int kFusedMaxTiles = DLB_WS_COUNTER_BYTES / 16;  // four counter words per tile in the workspace head
 
 // Raise a kernel's dynamic LDS limit once per (kernel, device).
@@ -551,8 +553,9 @@ struct Resolved {
   bool fused;                // K slices added inside the launch (counters in the workspace head), no second pass
 };
 
+// fused_act: the launch is one of the gate/up GEMMs with the activation in its epilogue (their kernels take no scale table)
 Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as_sm, int64_t as_sk, bool have_ws,
-                 size_t ws_bytes, int cus, bool gather_scales = false) {
+                 size_t ws_bytes, int cus, bool gather_scales = false, bool fused_act = false) {
   Resolved r{};
   const int64_t kblocks = ceil_div(K, kScaleBlock);
   const int64_t groups = mode == kMasked ? G : 1;  // a_s is per expert only in the masked layout; contiguous rows are one matrix
@@ -572,8 +575,11 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
   // Small ring kernels with at most 32 K blocks per workgroup fetch a tile's row-major scales once, into a table in
   // LDS: no re-layout pass, one cache-line request per row and tile.
   const bool small_ring = pl.variant == kVarPipe128x128 || pl.variant == kVarPipe128x64;
+  // (the masked layout's 128 x 256 tiles take the table too: a decode-sized K, no re-layout launch in front)
+  const bool masked_ring = mode == kMasked && pl.variant == kVarPipe128x256w8 && !gather_scales && !fused_act && g_forced_variant < 0;
   auto table_fits = [&](int kb_per) {
-    return mode == kDense && small_ring && g_knob[kKnobScaleTable] != 2 && as_sm != 1 && kb_per <= 32 && as_sk < (1ll << 20) && dma_ok;
+    return ((mode == kDense && small_ring) || masked_ring) && g_knob[kKnobScaleTable] != 2 && as_sm != 1 &&
+           kb_per <= (masked_ring ? Pipe128x256w8T::SCTAB_KB : Pipe128x64T::SCTAB_KB) && as_sk < (1ll << 20) && dma_ok;
   };
   r.sctab = table_fits(r.kb_per_split);
   // gather_scales: the re-layout pass also brings the rows into the GEMM's order, so it runs whatever the strides
@@ -711,7 +717,7 @@ int run(const Problem& pr) {
 
   if (pr.ws && misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
   const Resolved rs = resolve(pr.mode, pr.rows, pr.N, pr.K, pr.G, pr.as_sm, pr.as_sk, pr.ws != nullptr, pr.ws_bytes, cus,
-                              pr.a_rows != nullptr);
+                              pr.a_rows != nullptr, pr.act);
   const Plan& pl = rs.pl;
   // everything that can refuse the launch is checked before the first pre-pass kernel is enqueued
   if (rs.grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)rs.grid);
@@ -849,6 +855,7 @@ int run(const Problem& pr) {
     }
     if (pl.variant == kVarPipe128x256w8 && pr.act)
       return launch_pipelined<Pipe128x256w8, kMaskedAct>(ar, g, dev, pr.stream);  // N / 256 column tiles, as the plain GEMM
+    if (pl.variant == kVarPipe128x256w8 && pr.mode == kMasked && rs.sctab) return launch_pipelined<Pipe128x256w8T, kMasked>(ar, g, dev, pr.stream);
     if (pl.variant == kVarPipe128x256w8) return launch_pipelined_mode<Pipe128x256w8>(pr.mode, ar, g_dense, dev, pr.stream);
     if (pl.variant == kVarPipe128x128)
       return rs.sctab ? launch_pipelined<Pipe128x128T, kDense>(ar, g, dev, pr.stream)

@@ -106,7 +106,7 @@ __device__ __forceinline__ v4f coherent_load16(const float* src) {
 // SCTAB_: true = the activation scales of a tile's rows for ALL K blocks of the workgroup's K range (at most
 // SCTAB_KB) are fetched once per tile into a table behind the ring, lanes along K: a row-major a_s then costs one
 // cache-line request per row and tile instead of one per row and K step, and needs no re-layout pass in front.
-template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_, int PARTS_ = 2, bool PREFETCH_ = false, bool SCTAB_ = false>
+template <int WGM_, int WGN_, int MF_, int NF_, int STAGES_, int PARTS_ = 2, bool PREFETCH_ = false, bool SCTAB_ = false, int SCTAB_KB_ = 32>
 struct PipeCfg {
   static constexpr int WGM = WGM_, WGN = WGN_, MF = MF_, NF = NF_, STAGES = STAGES_, PARTS = PARTS_;
   static constexpr bool PREFETCH = PREFETCH_;
@@ -124,7 +124,7 @@ struct PipeCfg {
   static constexpr int S_BYTES = S_INST * NT * 4;  // activation scales of the tile rows for one K block
   static constexpr int W_BYTES = NT * 4;           // weight scale of each wave's n block, one copy per lane
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + S_BYTES + W_BYTES;
-  static constexpr int SCTAB_KB = 32;              // K blocks per workgroup the table holds
+  static constexpr int SCTAB_KB = SCTAB_KB_;       // K blocks per workgroup the table holds
   static constexpr int SCTAB_OFF = STAGES * STAGE_BYTES;
   static constexpr int SCTAB_BYTES = SCTAB ? BM * SCTAB_KB * 4 : 0;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + SCTAB_BYTES;

@@ -475,6 +475,42 @@ def test_grouped_masked(dev):
     helpers.tolerance_check(out, ref, 'grouped masked')
 
 
+@pytest.mark.parametrize('K', [384, 2048, 2176])
+def test_grouped_masked_scale_table(dev, K):
+    """The masked layout fetches a tile's row-major activation scales once, into a table in LDS, when K has at most 16
+    blocks (no re-layout launch in front); longer K and the knob take the re-laid copy in the workspace.  Same bits
+    either way, rows at or beyond masked_m (NaN codes, NaN scales) never read into a valid row nor written."""
+    from dlblas_amd import _lib
+    from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
+    print(f'case masked scale table K={K}', flush=True)
+    G, M_max, N = 5, 256, 512
+    g = helpers.gen(14)
+    masked_m = torch.tensor([3, 256, 0, 129, 200], dtype=torch.int32)
+    a_q, a_s = orc.quant_act_1x128(torch.randn(G, M_max, K, generator=g).to(torch.bfloat16))
+    w_q, w_s = _make_grouped_weights(G, N, K, 15)
+    a_bits = a_q.view(torch.uint8).clone()
+    for e in range(G):
+        a_bits[e, int(masked_m[e]):] = 0x7F
+        a_s[e, int(masked_m[e]):] = float('nan')
+    a_q = a_bits.view(torch.float8_e4m3fn)
+    sentinel = -555.0
+    ref = orc.grouped_masked_ref(a_q, a_s, w_q, w_s, torch.full((G, M_max, N), sentinel), masked_m)
+    outs = []
+    for knob in (0, 2):
+        out = torch.full((G, M_max, N), sentinel, dtype=torch.bfloat16, device=dev)
+        _lib.tune('scale_table', knob)
+        try:
+            m_grouped_fp8_gemm_nt_masked((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, masked_m.to(dev), 128)
+            torch.cuda.synchronize()
+        finally:
+            _lib.tune('scale_table', 0)
+        outs.append(out)
+    for e in range(G):
+        assert torch.all(outs[0][e, int(masked_m[e]):] == sentinel)
+    helpers.tolerance_check(outs[0], ref, f'masked scale table K={K}')
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_registry_selects_and_caches_on_gpu(dev):
     print('case registry', flush=True)
     from dlblas_amd import get_op
