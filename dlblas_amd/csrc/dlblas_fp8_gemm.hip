@@ -306,11 +306,15 @@ double mixed_makespan(int64_t ta, int64_t tb, double cb, int workers) {
 
 // Columns [0, n_split) in 256-wide tiles, the rest in 192-wide tiles; returns n_split (== N: no narrow region).
 // Cost: (N / 256 + 1) candidate cuts x a few steps per round, a few microseconds at most, no state.
-int64_t pick_mixed_split(int64_t M, int64_t N, int cus) {
+// *makespan (optional): the launch's length in units of one 256-wide tile.
+int64_t pick_mixed_split(int64_t M, int64_t N, int cus, double* makespan = nullptr) {
   const int64_t tm = ceil_div(M, 256);
   const double narrow_cost = 0.78;  // 192 / 256 of the work plus the fixed per-tile part
   int64_t best_split = N;
-  if (tm * ceil_div(N, 256) > 16 * static_cast<int64_t>(cus)) return N;  // many rounds: the tail no longer matters
+  if (tm * ceil_div(N, 256) > 16 * static_cast<int64_t>(cus)) {  // many rounds: the tail no longer matters
+    if (makespan) *makespan = static_cast<double>(ceil_div(tm * ceil_div(N, 256), cus));
+    return N;
+  }
   const double uniform = mixed_makespan(tm * ceil_div(N, 256), 0, narrow_cost, cus);
   double best = uniform;
   for (int64_t ca = N / 256; ca >= 0; --ca) {
@@ -319,7 +323,25 @@ int64_t pick_mixed_split(int64_t M, int64_t N, int cus) {
     const double t = mixed_makespan(tm * ca, tm * ceil_div(N - split, 192), narrow_cost, cus);
     if (t < best - 1e-6 && t < 0.96 * uniform) best = t, best_split = split;  // a uniform launch of many rounds runs resident, worth 4 %
   }
+  if (makespan) *makespan = best;
   return best_split;
+}
+
+// Prefill-sized dense problems: 256-row tiles (256 and 192 columns wide, mixed so that the rounds come out even) or
+// 128 x 256 tiles?  Both run from the L2 at the pace of the matrix pipe there - 1.62 us per K step of a 256 x 256 tile,
+// 1.0 us for 128 x 256 - and a tile costs a fixed 11.5 / 5.5 us on top (its first loads, its output; 4.3 us in a launch
+// of four rounds or more, which runs as resident workgroups; measured on MI355X, 192 ... 4096 rows, K = 512 ... 18432).
+// The larger tile wins unless its rows are mostly padding (384 rows are two 256-row tiles but three of 128), its tiles
+// leave much of a round empty (2048 x 4096: 128 tiles of 256 x 256 on 256 CUs, but 256 tiles of 128 x 256), or K is so
+// short that the fixed part decides: 384 x 18432 x 7168 82 -> 67 us, 2048 x 4096 x 7168 79 -> 67 us,
+// 4096 x 32768 x 512 166 -> 155 us.
+bool prefers_128_row_tiles(int64_t M, int64_t N, int kblocks, int cus) {
+  double span = 0.0;
+  pick_mixed_split(M, N, cus, &span);
+  const double wide_us = span * (11.5 + 1.62 * kblocks);
+  const int64_t rounds = ceil_div(ceil_div(M, 128) * ceil_div(N, 256), cus);
+  const double half_us = static_cast<double>(rounds) * ((rounds >= 4 ? 4.3 : 5.5) + 1.0 * kblocks);
+  return half_us < 0.95 * wide_us;
 }
 
 struct Plan {
@@ -453,8 +475,8 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
       if (M > 64 && kblocks >= 32 && ceil_div(N, 128) * 2 <= cus) v = kVarTile128x128;
       if (M > 32 && whole_blocks) {
         // 33 .. 128 rows: the streaming kernel costs what is larger of its workgroups each reading all activation rows
-        // from the L2 (about 6.5 TB/s over the chip) and of its waves' K blocks, fetched one after the other: a round
-        // of 8 blocks lasts 0.14 us + 24 ns per activation row + 40 ns per weight row of the workgroup (measured at
+        // from the L2 (about 8.5 TB/s over the chip) and of its waves' K blocks, fetched one after the other: a round
+        // of 8 blocks lasts 0.8 x (0.14 us + 24 ns per activation row + 40 ns per weight row of the workgroup) (measured at
         // 33 .. 128 rows, 4 .. 28 weight rows, K = 2048 .. 16384).  A K-split tile kernel wins when the weight matrix
         // is narrow and K long (2112 x 7168: 18.3 -> 14.1 us at 64 rows, 29 -> 17.4 us at 128; at 33 rows the streaming
         // kernel stays ahead, 11.9 against 13.2 us)
@@ -463,8 +485,8 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
         const int64_t wgs = ceil_div(N, bn);
         const double m_eff = M <= 64 ? static_cast<double>(M) : 0.5 * (M + 128.0);  // the 128-row kernel computes all 8 row fragments
         const double round_us = 0.14 + 0.0239 * m_eff + 0.04 * bn;
-        const double chain_us = round_us * static_cast<double>(ceil_div(kblocks, 8)) * static_cast<double>(ceil_div(wgs, cus));
-        const double l2_us = static_cast<double>(wgs) * M * K / 6.5e6;
+        const double chain_us = 0.8 * round_us * static_cast<double>(ceil_div(kblocks, 8)) * static_cast<double>(ceil_div(wgs, cus));
+        const double l2_us = static_cast<double>(wgs) * M * K / 8.5e6;
         const double stream_us = 2.6 + (l2_us > chain_us ? l2_us : chain_us);
         const MidChoice mid = pick_mid_plan(M, N, kblocks, cus, ws_avail);
         if (mid.us < stream_us) v = mid.variant, mid_splitk = mid.splitk;
@@ -473,7 +495,7 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
     } else if (whole_blocks && mode == kDense) {
       const int64_t t256 = ceil_div(M, 256) * ceil_div(N, 256);
       if (t256 * 2 >= cus) {
-        v = kVarPipe256mix;
+        v = prefers_128_row_tiles(M, N, kblocks, cus) ? kVarPipe128x256w8 : kVarPipe256mix;
       } else {
         const MidChoice mid = pick_mid_plan(M, N, kblocks, cus, ws_avail);
         v = mid.variant, mid_splitk = mid.splitk;

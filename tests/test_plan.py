@@ -35,6 +35,13 @@ def test_documented_choices():
     v, s, _ = _lib.plan(DENSE, 256, 7168, 16384)
     assert v in RING and s > 1
     assert _lib.plan(DENSE, 256, 7168, 2048) == ('pipe128x64', 1, 0)
+    # prefill-sized: 256-row tiles unless their rows are mostly padding, they leave a round half empty or K is short
+    assert _lib.plan(DENSE, 512, 18432, 7168) == ('pipe256mix', 1, 0)
+    assert _lib.plan(DENSE, 384, 18432, 7168) == ('pipe128x256w8', 1, 0)  # two 256-row tiles, but three of 128 rows
+    assert _lib.plan(DENSE, 2048, 4096, 7168) == ('pipe128x256w8', 1, 0)  # 128 tiles of 256 x 256 on 256 CUs
+    assert _lib.plan(DENSE, 4096, 4096, 7168) == ('pipe256mix', 1, 0)
+    assert _lib.plan(DENSE, 4096, 32768, 512) == ('pipe128x256w8', 1, 0)  # four K blocks: the tile's fixed part decides
+    assert _lib.plan(DENSE, 48, 4096, 7168)[0] == 'skinny64'             # few rows stream even a narrow weight matrix
     assert _lib.plan(DENSE, 17, 64, 200)[0] == 'exact'                   # K % 16 != 0
     assert _lib.plan(DENSE, 300, 200, 400)[0] == 'tile128x128'           # K tail: the register-staged kernel
     assert _lib.plan(CONTIGUOUS, 9728, 4096, 7168) == ('pipe128x256w8', 1, 0)
