@@ -35,6 +35,9 @@ WORKLOADS = {
 }
 # measured after the timed region and reported under "other_workloads" (name: M, N, K)
 DECODE_SWEEP = [(m, n, k) for (n, k) in ((7168, 2048), (2112, 7168)) for m in (1, 16, 64, 128)]
+# the dense MLP's projections of the same model at 16 rows: weight matrices large enough that the launch is not
+# most of the time (132 and 264 MB)
+DECODE_SWEEP += [(16, 7168, 18432), (16, 36864, 7168)]
 GROUPED_CONTIGUOUS = dict(G=32, tokens=8192, N=4096, K=7168)
 GROUPED_MASKED = dict(G=32, M_max=256, N=7168, K=2048)
 
@@ -224,13 +227,17 @@ def time_call(fn, iters, warmup):
 
 
 def decode_sweep(dev):
-    """HBM-bound shapes: 24 distinct weight copies in rotation (> 256 MB) so that reads come from HBM."""
+    """HBM-bound shapes: distinct weight copies in rotation (24 of the small matrices, > 256 MB in all) so that reads
+    come from HBM."""
     import torch
     rows = []
     for (M, N, K) in DECODE_SWEEP:
-        a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=24)
+        copies = max(2, min(24, -(-400_000_000 // (N * K))))
+        a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=copies)
         out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-        ms = time_call(DenseLauncher(a_q, a_s, ws, out), 480, 1500)  # 1500 untimed launches (~10 ms): clocks at their loaded level
+        small = N * K < 50_000_000
+        # 1500 untimed launches of a small matrix (~10 ms): clocks at their loaded level
+        ms = time_call(DenseLauncher(a_q, a_s, ws, out), 480 if small else 120, 1500 if small else 300)
         nbytes = algorithmic_bytes(M, N, K)
         rows.append({'workload': f'decode_{M}x{N}x{K}', 'us_per_launch': ms * 1e3, 'GBps': nbytes / ms / 1e6,
                      'frac_of_hbm_peak': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'TFLOPs': 2.0 * M * N * K / ms / 1e9,
