@@ -12,7 +12,7 @@ import torch
 
 from ._build import LIB_PATH
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 OUT_BF16, OUT_F32 = 0, 1
 WS_COUNTER_BYTES = 65536
 WORKSPACE_BYTES = WS_COUNTER_BYTES + (32 << 20)
@@ -50,6 +50,8 @@ SYMBOLS = {
     'dlb_fp8_gemm_variant_name': (ctypes.c_char_p, [ctypes.c_int]),
     'dlb_fp8_gemm_plan': (ctypes.c_int, [ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_sz, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 3 +
                           [ctypes.POINTER(_c_i64)]),
+    'dlb_fp8_gemm_plan_grouped': (ctypes.c_int, [ctypes.c_int, _c_i64, _c_i64, _c_i64, ctypes.c_int32, ctypes.c_int32, _c_sz, ctypes.c_int,
+                                                ctypes.POINTER(ctypes.c_int)]),
     'dlb_silu_mul': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp] + [_c_i64] * 4 + [_c_vp]),
     'dlb_silu_mul_quant': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
     'dlb_silu_mul_quant_masked': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp, _c_vp] + [_c_i64] * 6 + [_c_vp]),
@@ -181,6 +183,16 @@ def plan_full(mode: int, rows: int, N: int, K: int, workspace_bytes: int = None,
     return variant_names()[v.value], s.value, c.value, n.value
 
 
+def plan_grouped(mode: int, rows: int, N: int, K: int, G: int, expected_m: int = -1, workspace_bytes: int = None,
+                 compute_units: int = 256):
+    """(variant name,) of a grouped launch (mode 1 contiguous, 2 masked) with G experts and the masked layout's hint."""
+    lib = load()
+    v = ctypes.c_int()
+    ws = WORKSPACE_BYTES if workspace_bytes is None else workspace_bytes
+    check(lib.dlb_fp8_gemm_plan_grouped(mode, rows, N, K, G, expected_m, ws, compute_units, ctypes.byref(v)))
+    return (variant_names()[v.value], )
+
+
 def force_variant(name_or_id) -> None:
     """Pin the kernel variant used by later calls from this thread (None or -1: back to the heuristic)."""
     lib = load()
@@ -192,7 +204,7 @@ def force_variant(name_or_id) -> None:
 
 
 KNOBS = {'splitk': 0, 'skinny_waves': 1, 'skinny_unroll': 2, 'skinny_nfrags': 3, 'group_m': 4, 'skinny_dma': 5, 'epilogue': 6, 'skinny_bn': 7,
-         'splitk_mode': 8, 'spin_limit': 9, 'scale_table': 10, 'lds_oversize': 11, 'masked_grid': 12}
+         'splitk_mode': 8, 'spin_limit': 9, 'scale_table': 10, 'lds_oversize': 11, 'masked_grid': 12, 'tile_list': 13}
 
 
 def tune(knob: str, value) -> None:

@@ -98,9 +98,10 @@ enum Knob : int {
   kKnobScaleTable, // 0 / 1: row-major activation scales of the small ring kernels go through the per-tile table, 2: never
   kKnobLdsOversize,  // test hook: 1 = ask for more LDS than the GPU has, so that the launch is refused before anything is enqueued
   kKnobMaskedGrid,   // workgroups per CU of the masked layout's persistent grid (0 = default)
+  kKnobTileList,     // expert-contiguous rows: 1 = device-built tile lists whenever possible, 2 = never (0 = by batch size)
   kKnobCount
 };
-thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+thread_local int g_knob[kKnobCount] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 // set while run() asks every kernel of the call for its launch attributes, before the first pre-pass is enqueued
 thread_local bool g_prepare_only = false;
 constexpr int kDefaultSpinLimit = 400;  // x about 0.5 us: far beyond the spread of the slices of one round of workgroups
@@ -456,7 +457,10 @@ MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_av
 
 // dma_ok: the DMA kernels address their sources with 32-bit byte offsets from the tile's first row (up to 256 rows x K
 // bytes, 512 scale rows x stride); false sends such problems to the kernels with 64-bit addressing.
-Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes, bool dma_ok) {
+// G, hint_rows (grouped layouts): experts, and the masked layout's typical rows per expert (<= 0: unknown).
+// fixed_grouped: the caller needs the 128 x 256 kernel (the fused activation epilogues exist for it only).
+Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_bytes, bool dma_ok, int G = 1,
+               int64_t hint_rows = -1, bool fixed_grouped = false) {
   Plan pl{kVarTile128x128, 128, 128, 1, 4, 4, 1, 16, dma_ok};
   const int kblocks = static_cast<int>(ceil_div(K, kScaleBlock));
   const size_t ws_avail = ws_bytes > DLB_WS_COUNTER_BYTES ? ws_bytes - DLB_WS_COUNTER_BYTES : 0;
@@ -502,6 +506,23 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
       }
     } else if (whole_blocks) {
       v = kVarPipe128x256w8;  // grouped: 128-row tiles never straddle two experts / waste at most 127 masked rows
+      const int64_t tn = ceil_div(N, 256);
+      if (fixed_grouped || (mode == kContiguous && g_knob[kKnobTileList] == 1)) {
+      } else if (mode == kContiguous) {
+        // a small batch: 128 x 128 tiles while 128 x 256 ones would leave half the CUs idle
+        // (8 experts x 128 rows x 4096 x 7168: 67 -> 54 us)
+        if (ceil_div(M, 128) * tn * 2 <= cus) v = kVarPipe128x128;
+      } else if (hint_rows > 0) {
+        // masked, with the caller's hint: few rows per expert and few experts - smaller tiles, as above (8 experts,
+        // 4096 x 7168, up to 128 rows each: 54 - 75 -> 44 - 55 us); several hundred rows per expert - 256-row tiles,
+        // which fetch an expert's weights once per 256 rows (32 experts x ~520 rows x 4096 x 7168: 665 -> 573 us,
+        // 7168 x 2048: 363 -> 335 us)
+        // (or two 128-row tiles per expert that fill one round at most: 8 experts x ~240 rows: 121 -> 110 us)
+        const int64_t em = hint_rows < M ? hint_rows : M;
+        const int64_t units = static_cast<int64_t>(G) * ceil_div(em, 128) * tn;
+        if (units * 2 <= cus) v = kVarPipe128x128;
+        else if (em >= 384 || (em >= 192 && units <= cus)) v = kVarPipe256x256;
+      }
     } else {
       v = (M <= 64 && mode != kContiguous) ? kVarTile64x128 : kVarTile128x128;
     }
@@ -583,13 +604,13 @@ struct Resolved {
 
 // fused_act: the launch is one of the gate/up GEMMs with the activation in its epilogue (their kernels take no scale table)
 Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as_sm, int64_t as_sk, bool have_ws,
-                 size_t ws_bytes, int cus, bool gather_scales = false, bool fused_act = false) {
+                 size_t ws_bytes, int cus, bool gather_scales = false, bool fused_act = false, int64_t hint_rows = -1) {
   Resolved r{};
   const int64_t kblocks = ceil_div(K, kScaleBlock);
   const int64_t groups = mode == kMasked ? G : 1;  // a_s is per expert only in the masked layout; contiguous rows are one matrix
   const bool dma_ok = K < (1ll << 24) && as_sm < (1ll << 21);
   const bool usable_ws = have_ws && ws_bytes > DLB_WS_COUNTER_BYTES;
-  r.pl = make_plan(mode, rows, N, K, cus, usable_ws ? ws_bytes : 0, dma_ok);
+  r.pl = make_plan(mode, rows, N, K, cus, usable_ws ? ws_bytes : 0, dma_ok, G, hint_rows, fused_act || gather_scales);
   const Plan& pl = r.pl;
   const int want = usable_ws ? pl.splitk : 1;
   r.kb_per_split = static_cast<int>(ceil_div(kblocks > 0 ? kblocks : 1, want));
@@ -598,7 +619,12 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
   if (mode == kContiguous && pl.variant == kVarPipe128x256w8 && g_forced_variant < 0 && usable_ws && kblocks > 0) {
     const int64_t nblk = ceil_div(rows, kScaleBlock);
     const size_t bytes = tile_list_bytes(nblk);
-    if (nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
+    // Taller tiles save weight traffic, not time per tile: while two rounds of 128-row tiles cover the batch, those
+    // are faster and need no list (8 experts, 1408 rows, 4096 x 7168: 107 -> 69 us; 32 experts x 128 rows: 183 ->
+    // 174 us).  The fused epilogues exist for the list kernel only.
+    const bool worth_it = fused_act || gather_scales || g_knob[kKnobTileList] == 1 ||
+                          (g_knob[kKnobTileList] != 2 && nblk * ceil_div(N, 256) > 2ll * cus);
+    if (worth_it && nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
   }
   // Small ring kernels with at most 32 K blocks per workgroup fetch a tile's row-major scales once, into a table in
   // LDS: no re-layout pass, one cache-line request per row and tile.
@@ -687,6 +713,7 @@ struct Problem {
   int64_t a_src_rows = 0;
   float act_eps = 0.f;
   bool act = false;
+  int64_t hint_rows = -1;  // masked layout: the caller's expected_m
 };
 
 
@@ -745,7 +772,7 @@ int run(const Problem& pr) {
 
   if (pr.ws && misaligned(pr.ws, 16)) return fail(DLB_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
   const Resolved rs = resolve(pr.mode, pr.rows, pr.N, pr.K, pr.G, pr.as_sm, pr.as_sk, pr.ws != nullptr, pr.ws_bytes, cus,
-                              pr.a_rows != nullptr, pr.act);
+                              pr.a_rows != nullptr, pr.act, pr.hint_rows);
   const Plan& pl = rs.pl;
   // everything that can refuse the launch is checked before the first pre-pass kernel is enqueued
   if (rs.grid > (1ll << 30)) return fail(DLB_ERR_BAD_SHAPE, "too many tiles (%lld)", (long long)rs.grid);
@@ -1133,9 +1160,9 @@ int dlb_fp8_gemm_grouped_masked(const void* a, const void* b, const float* a_s, 
                                 const int32_t* masked_m, int32_t expected_m, int64_t M_max, int64_t N, int64_t K,
                                 int32_t G, int64_t as_stride_g, int64_t as_stride_m, int64_t as_stride_k,
                                 int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
-  (void)expected_m;
   dlb::Problem pr{dlb::kMasked, a, b, a_s, b_s, c, masked_m, M_max, N, K, G, as_stride_g, as_stride_m, as_stride_k,
                   out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+  pr.hint_rows = expected_m;
   return dlb::run(pr);
 }
 
@@ -1233,6 +1260,20 @@ int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t works
   if (k_slices) *k_slices = rs.splitk;
   if (decode_columns) *decode_columns = dlb::is_skinny(rs.pl.variant) ? rs.pl.sk_bn : 0;
   if (narrow_from) *narrow_from = rs.n_split;
+  return DLB_OK;
+}
+
+int dlb_fp8_gemm_plan_grouped(int mode, int64_t rows, int64_t N, int64_t K, int32_t G, int32_t expected_m, size_t workspace_bytes,
+                              int compute_units, int* variant) {
+  dlb::clear_error();
+  if (mode != dlb::kContiguous && mode != dlb::kMasked) return dlb::fail(DLB_ERR_BAD_SHAPE, "mode %d is not 1 (contiguous) or 2 (masked)", mode);
+  if (rows < 0 || N < 0 || K < 0 || G < 0) return dlb::fail(DLB_ERR_BAD_SHAPE, "negative dimension (rows=%lld, N=%lld, K=%lld, G=%d)", (long long)rows, (long long)N, (long long)K, G);
+  const int64_t lim = (1ll << 31) - 1024;
+  if (rows > lim || N > lim || K > lim) return dlb::fail(DLB_ERR_BAD_SHAPE, "dimension beyond 2^31");
+  if (compute_units <= 0) return dlb::fail(DLB_ERR_BAD_SHAPE, "compute_units must be positive");
+  const dlb::Resolved rs = dlb::resolve(mode, rows, N, K, G, dlb::ceil_div(K, dlb::kScaleBlock), 1, workspace_bytes > 0, workspace_bytes,
+                                        compute_units, false, false, mode == dlb::kMasked ? expected_m : -1);
+  if (variant) *variant = rs.pl.variant;
   return DLB_OK;
 }
 

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define DLB_ABI_VERSION 6
+#define DLB_ABI_VERSION 7
 
 /* output element type of C */
 #define DLB_OUT_BF16 0
@@ -212,7 +212,10 @@ int dlb_fp8_gemm_grouped_contiguous_gather_silu_quant(const void* a, const void*
  *                                             are computed; rows at or beyond it are neither read
  *                                             into a valid result nor written.  Values are clamped
  *                                             to [0, M_max].
- *   expected_m                                scheduling hint only (typical masked_m); <= 0 = unknown
+ *   expected_m                                scheduling hint only (typical masked_m); <= 0 = unknown.
+ *                                             It picks the tile shape (128 x 128 for a few short experts,
+ *                                             256-row tiles from several hundred rows per expert on) and
+ *                                             never changes a result bit.
  *
  * The tile schedule is built on the device from masked_m: no host synchronisation and no tiles
  * for empty row ranges.  K % 16 == 0 is required.
@@ -308,6 +311,14 @@ int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t works
                       int* k_slices, int* decode_columns, int64_t* narrow_from);
 
 /*
+ * The same query for the grouped layouts with what their choice depends on besides the shape: the expert count and, for
+ * the masked layout (mode 2), the caller's expected_m (<= 0: unknown).  mode 1 = contiguous (rows = M_sum), 2 = masked
+ * (rows = M_max).  No counterpart in the reference.
+ */
+int dlb_fp8_gemm_plan_grouped(int mode, int64_t rows, int64_t N, int64_t K, int32_t G, int32_t expected_m, size_t workspace_bytes,
+                              int compute_units, int* variant);
+
+/*
  * Tuning / test hook: force the kernel variant the next calls FROM THIS THREAD use.
  * variant < 0 restores the built-in shape heuristic.  Returns DLB_ERR_BAD_SHAPE for an unknown id.
  * Variant ids are listed by dlb_fp8_gemm_variant_name().
@@ -335,6 +346,9 @@ int dlb_fp8_gemm_force_variant(int variant);
  *   DLB_KNOB_SCALE_TABLE    2 = the small DMA-ring kernels fetch row-major activation scales stage by stage instead of
  *                           once per tile into a table in LDS
  *   DLB_KNOB_MASKED_GRID    workgroups per CU of the persistent grid of the masked layout (default 1)
+ *   DLB_KNOB_TILE_LIST      expert-contiguous rows: 1 = 256- / 192- / 128-row tiles from lists built on the device
+ *                           whenever a workspace allows it, 2 = uniform 128-row tiles (default: lists from more than two
+ *                           rounds of 128 x 256 tiles on)
  *   DLB_KNOB_LDS_OVERSIZE   test hook: 1 = every kernel asks for more LDS than the GPU has, so the call is refused
  *                           (DLB_ERR_LAUNCH) before anything is enqueued
  */
@@ -351,6 +365,7 @@ int dlb_fp8_gemm_force_variant(int variant);
 #define DLB_KNOB_SCALE_TABLE 10
 #define DLB_KNOB_LDS_OVERSIZE 11
 #define DLB_KNOB_MASKED_GRID 12
+#define DLB_KNOB_TILE_LIST 13
 int dlb_fp8_gemm_tune(int knob, int value);
 
 /* Name of kernel variant `variant`, or NULL beyond the last one. */

@@ -394,11 +394,12 @@ def test_grouped_contiguous(dev, col_major_scales, out_dtype):
     helpers.tolerance_check(out, ref, 'grouped contiguous')
 
 
-@pytest.mark.parametrize('variant', [None, 'pipe128x256w8', 'tile128x128'])
+@pytest.mark.parametrize('variant', [None, 'list', 'pipe128x256w8', 'tile128x128'])
 def test_grouped_contiguous_run_lengths(dev, variant):
     """Runs of 1 to 5 blocks of 128 rows, skipped blocks between and inside runs, an expert that owns two separate
-    runs, experts out of order: the library's own choice pairs blocks into 256-row tiles from a list built on the
-    device; forced variants take the uniform 128-row path.  All must agree with the oracle."""
+    runs, experts out of order.  'list' pairs blocks into 256-row tiles from a list built on the device (the library's
+    own choice for batches of more than two rounds of tiles; a batch this small gets 128 x 128 tiles); forced variants
+    take the uniform 128-row path.  All must agree with the oracle."""
     print(f'case contiguous run lengths variant={variant}', flush=True)
     from dlblas_amd import _lib
     from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_contiguous
@@ -413,11 +414,16 @@ def test_grouped_contiguous_run_lengths(dev, variant):
     ref = orc.grouped_contiguous_ref(a_q, a_s, w_q, w_s, torch.full((M_sum, N), sentinel), m_indices)
     out = torch.full((M_sum, N), sentinel, dtype=torch.bfloat16, device=dev)
     try:
-        _lib.force_variant(variant)
+        if variant == 'list':
+            _lib.tune('tile_list', 1)
+            assert _lib.plan(1, M_sum, N, K)[0] == 'pipe128x256w8'
+        else:
+            _lib.force_variant(variant)
         m_grouped_fp8_gemm_nt_contiguous((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, m_indices.to(dev))
         torch.cuda.synchronize()
     finally:
         _lib.force_variant(None)
+        _lib.tune('tile_list', 0)
     skipped = (m_indices < 0)
     assert torch.all(out.cpu()[skipped] == sentinel), 'a skipped block was written'
     helpers.tolerance_check(out, ref, f'contiguous run lengths {variant}')
@@ -467,12 +473,44 @@ def test_grouped_masked(dev):
     sentinel = -555.0
     ref = orc.grouped_masked_ref(a_q, a_s, w_q, w_s, torch.full((G, M_max, N), sentinel), masked_m)
     out = torch.full((G, M_max, N), sentinel, dtype=torch.bfloat16, device=dev)
-    m_grouped_fp8_gemm_nt_masked((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, masked_m.to(dev), 128)
+    m_grouped_fp8_gemm_nt_masked((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, masked_m.to(dev), 0)
     torch.cuda.synchronize()
     for e in range(G):
         assert torch.all(out[e, int(masked_m[e]):] == sentinel), f'expert {e}: rows beyond masked_m were written'
     assert not torch.isnan(out.float()).any()
     helpers.tolerance_check(out, ref, 'grouped masked')
+
+
+def test_grouped_masked_hint_picks_the_tile_shape(dev):
+    """expected_m picks the tile shape - unknown: 128 x 256; a few short experts: 128 x 128; several hundred rows per
+    expert: 256-row tiles - and never a result bit."""
+    print('case masked expected_m', flush=True)
+    from dlblas_amd import _lib
+    from dlblas_amd.kernels.fp8_gemm_grouped import m_grouped_fp8_gemm_nt_masked
+    G, M_max, N, K = 6, 512, 1536, 256
+    g = helpers.gen(16)
+    masked_m = torch.tensor([0, 1, 512, 130, 400, 257], dtype=torch.int32)
+    a_q, a_s = orc.quant_act_1x128(torch.randn(G, M_max, K, generator=g).to(torch.bfloat16))
+    w_q, w_s = _make_grouped_weights(G, N, K, 17)
+    a_bits = a_q.view(torch.uint8).clone()
+    for e in range(G):
+        a_bits[e, int(masked_m[e]):] = 0x7F
+        a_s[e, int(masked_m[e]):] = float('nan')
+    a_q = a_bits.view(torch.float8_e4m3fn)
+    sentinel = -555.0
+    ref = orc.grouped_masked_ref(a_q, a_s, w_q, w_s, torch.full((G, M_max, N), sentinel), masked_m)
+    outs, shapes = [], []
+    for hint in (0, 16, 500):
+        shapes.append(_lib.plan_grouped(2, M_max, N, K, G, hint)[0])
+        out = torch.full((G, M_max, N), sentinel, dtype=torch.bfloat16, device=dev)
+        m_grouped_fp8_gemm_nt_masked((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, masked_m.to(dev), hint)
+        torch.cuda.synchronize()
+        for e in range(G):
+            assert torch.all(out[e, int(masked_m[e]):] == sentinel), f'expected_m = {hint}, expert {e}: rows beyond masked_m were written'
+        outs.append(out)
+    assert shapes == ['pipe128x256w8', 'pipe128x128', 'pipe256x256'], shapes
+    helpers.tolerance_check(outs[0], ref, 'masked expected_m')
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
 
 
 @pytest.mark.parametrize('K', [384, 2048, 2176])
@@ -500,7 +538,7 @@ def test_grouped_masked_scale_table(dev, K):
         out = torch.full((G, M_max, N), sentinel, dtype=torch.bfloat16, device=dev)
         _lib.tune('scale_table', knob)
         try:
-            m_grouped_fp8_gemm_nt_masked((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, masked_m.to(dev), 128)
+            m_grouped_fp8_gemm_nt_masked((a_q.to(dev), a_s.to(dev)), (w_q.to(dev), w_s.to(dev)), out, masked_m.to(dev), 0)
             torch.cuda.synchronize()
         finally:
             _lib.tune('scale_table', 0)
