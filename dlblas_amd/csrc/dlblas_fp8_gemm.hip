@@ -442,8 +442,11 @@ MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_av
   // fewer rows than the 128 of a tile: the clamped rows repeat lines that are already on their way
   const double short_rows = M >= 128 ? 1.0 : 0.6 + 0.4 * static_cast<double>(M) / 128.0;
   for (const Cand& c : cands) {
-    for (int want : {1, 2, 3, 4, 5, 6, 7, 8}) {
+    for (int want : {1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16}) {
       if (want > 1 && (kblocks / want < 4 || out_bytes * want > static_cast<double>(ws_avail))) continue;
+      // more than 8 slices only while a slice keeps 8 K blocks (48 x 1024 x 16384: 17.9 -> 14.9 us with 16 slices;
+      // 64 x 576 x 7168: 11.0 -> 12.1 us with 14)
+      if (want > 8 && kblocks / want < 8) continue;
       const int per = static_cast<int>(ceil_div(kblocks, want));
       const int sk = static_cast<int>(ceil_div(kblocks, per));
       const int64_t units = ceil_div(M, c.bm) * ceil_div(N, c.bn) * sk;
