@@ -149,9 +149,10 @@ typedef PipeCfg<2, 2, 2, 2, DLB_EXP_P128, 2, false> Pipe128x128;  // experiment:
 typedef PipeCfg<2, 2, 2, 2, 4, 2, true> Pipe128x128;  // wave tile 64 x 64, 4 stages of 34 KB
 #endif
 typedef PipeCfg<2, 2, 2, 1, 5, 2, true> Pipe128x64;   // wave tile 64 x 32, 5 stages of 26 KB
-// the same with the activation scales of a tile in a table behind the ring (row-major a_s, at most 32 K blocks per workgroup)
-typedef PipeCfg<2, 2, 2, 2, 4, 2, true, true> Pipe128x128T;
-typedef PipeCfg<2, 2, 2, 1, 5, 2, true, true> Pipe128x64T;
+// the same with the activation scales of a tile in a table behind the ring (row-major a_s; as many K blocks per
+// workgroup as the LDS left by the ring holds: 54 and 64)
+typedef PipeCfg<2, 2, 2, 2, 4, 2, true, true, 54> Pipe128x128T;
+typedef PipeCfg<2, 2, 2, 1, 5, 2, true, true, 64> Pipe128x64T;
 typedef PipeCfg<2, 4, 2, 2, 3, 2, false, true, 16> Pipe128x256w8T;  // the masked layout's tiles (K of at most 16 blocks: 8 KB next to the 150 KB ring)
 static_assert(Pipe128x256w8T::LDS_BYTES <= 160 * 1024 && Pipe128x128T::LDS_BYTES <= 160 * 1024 && Pipe128x64T::LDS_BYTES <= 160 * 1024, "ring + table fit the LDS");
 constexpr int kFusedMaxTiles = DLB_WS_COUNTER_BYTES / 16;  // four counter words per tile in the workspace head
@@ -450,7 +451,11 @@ MidChoice pick_mid_plan(int64_t M, int64_t N, int kblocks, int cus, size_t ws_av
       const int per = static_cast<int>(ceil_div(kblocks, want));
       const int sk = static_cast<int>(ceil_div(kblocks, per));
       const int64_t units = ceil_div(M, c.bm) * ceil_div(N, c.bn) * sk;
-      double us = launch + relayout + static_cast<double>(ceil_div(units, cus)) * (tile_fixed + per * c.step_us * short_rows * scattered);
+      // the small tiles fetch a tile's scales once, into a table in LDS, when the slice is short enough: no re-layout
+      // launch and no scattered scale lines per K step
+      const bool table = (c.variant == kVarPipe128x64 && per <= Pipe128x64T::SCTAB_KB) || (c.variant == kVarPipe128x128 && per <= Pipe128x128T::SCTAB_KB);
+      double us = launch + (table ? 0.0 : relayout) +
+                  static_cast<double>(ceil_div(units, cus)) * (tile_fixed + per * c.step_us * short_rows * (table ? 1.0 : scattered));
       if (sk > 1) us += second_pass + (2.0 * sk + 0.5) * out_bytes / ws_rate;  // partial sums written, read back, result written
       if (us < best.us) best = MidChoice{c.variant, sk, us};
     }
@@ -601,7 +606,7 @@ struct Resolved {
   int64_t grid;              // workgroups of the main kernel
   bool resident;             // dense launch of many rounds: one resident workgroup per CU walks the tiles
   bool sctab;                // small ring kernels: row-major activation scales through the per-tile table in LDS
-  int sct_shift;             //   log2 of the table's row pitch
+  int sct_pitch;             //   floats per table row (odd)
   bool fused;                // K slices added inside the launch (counters in the workspace head), no second pass
 };
 
@@ -636,7 +641,9 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
   const bool masked_ring = mode == kMasked && pl.variant == kVarPipe128x256w8 && !gather_scales && !fused_act && g_forced_variant < 0;
   auto table_fits = [&](int kb_per) {
     return ((mode == kDense && small_ring) || masked_ring) && g_knob[kKnobScaleTable] != 2 && as_sm != 1 &&
-           kb_per <= (masked_ring ? Pipe128x256w8T::SCTAB_KB : Pipe128x64T::SCTAB_KB) && as_sk < (1ll << 20) && dma_ok;
+           kb_per <= (masked_ring ? Pipe128x256w8T::SCTAB_KB
+                                  : (pl.variant == kVarPipe128x64 ? Pipe128x64T::SCTAB_KB : Pipe128x128T::SCTAB_KB)) &&
+           as_sk < (1ll << 20) && dma_ok;
   };
   r.sctab = table_fits(r.kb_per_split);
   // gather_scales: the re-layout pass also brings the rows into the GEMM's order, so it runs whatever the strides
@@ -672,7 +679,7 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
   }
   if (r.sctab && !table_fits(r.kb_per_split)) r.sctab = false;  // fewer, longer slices than the table holds: scales in place
   if (r.sctab)
-    while ((1 << r.sct_shift) < r.kb_per_split) ++r.sct_shift;
+    r.sct_pitch = r.kb_per_split | 1;
   if (pl.variant == kVarPipe256mix) r.n_split = pick_mixed_split(rows, N, cus);
   const int64_t tiles_m = ceil_div(rows, pl.bm), tiles_n = ceil_div(N, pl.bn);
   int64_t grid = tiles_m * tiles_n * r.splitk;
@@ -848,7 +855,7 @@ int run(const Problem& pr) {
   hipError_t e = hipSuccess;
   ar.fused_reduce = rs.fused ? 1 : 0;
   ar.spin_limit = g_knob[kKnobSpinLimit] > 0 ? g_knob[kKnobSpinLimit] - 1 : kDefaultSpinLimit;
-  ar.sct_shift = rs.sct_shift;
+  ar.sct_pitch = rs.sct_pitch;
   const bool tile_list = rs.tile_list;
   const size_t esz = ar.out_f32 ? 4 : 2;
 

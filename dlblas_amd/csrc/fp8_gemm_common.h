@@ -55,7 +55,7 @@ struct Args {
   int kb_per_split;
   int fused_reduce;     // split-K in one launch: the workgroups of a tile add its K slices themselves (see splitk_fused_epilogue)
   int spin_limit;       //   polls (about half a microsecond apart) a workgroup waits for the other slices of its tile before it leaves its share to the last one
-  int sct_shift;        // kernels with a scale table in LDS: log2 of the table's row pitch (a power of two >= K blocks per workgroup)
+  int sct_pitch;        // kernels with a scale table in LDS: floats per table row (odd, >= K blocks per workgroup)
   int group_m;          // m-tiles per L2 swizzle group
   int out_f32;
   int vec_store;        // rows of c are aligned for 4-element vector stores

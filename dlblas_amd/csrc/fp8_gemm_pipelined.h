@@ -126,7 +126,7 @@ struct PipeCfg {
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + S_BYTES + W_BYTES;
   static constexpr int SCTAB_KB = SCTAB_KB_;       // K blocks per workgroup the table holds
   static constexpr int SCTAB_OFF = STAGES * STAGE_BYTES;
-  static constexpr int SCTAB_BYTES = SCTAB ? BM * SCTAB_KB * 4 : 0;
+  static constexpr int SCTAB_BYTES = SCTAB ? BM * (SCTAB_KB + 1) * 4 : 0;  // rows of an odd pitch (bank spread), at most SCTAB_KB + 1 floats
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + SCTAB_BYTES;
   static constexpr int LOADS_PER_STAGE = A_INST + B_INST + S_INST + 1;  // vmcnt units per wave and stage
   static_assert(BM % (8 * WAVES) == 0 && BN % (8 * WAVES) == 0, "tile rows must divide over the DMA instructions");
@@ -417,15 +417,19 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
 
     __syncthreads();  // the previous tile's readers and DMA groups are done with the ring
     if constexpr (Cfg::SCTAB) {
-      // scale table [BM][1 << sct_shift]: entry (r, j) = a_s of tile row r at the workgroup's j-th K block.  One DMA
+      // scale table [BM][p.sct_pitch]: entry (r, j) = a_s of tile row r at the workgroup's j-th K block.  One DMA
       // instruction moves 64 consecutive entries, i.e. whole runs of a row's scales; issued ahead of the first stages,
-      // so the wait for stage 0 covers them.
-      const int shift = p.sct_shift;
-      const int n_inst = (BM << shift) >> 6;
+      // so the wait for stage 0 covers them.  The pitch is odd: the 32 rows a wave reads at one K block then lie in 32
+      // different banks (with a power-of-two pitch of 32 floats they shared two banks, and every such read held the
+      // LDS for 16 turns while the other waves' fragment reads waited: 256 x 7168 x 4096 27.2 -> 24 us).
+      const int pitch = p.sct_pitch;
+      const float inv_pitch = 1.0f / static_cast<float>(pitch);
+      const int n_inst = (BM * pitch + 63) >> 6;
       for (int i = wave; i < n_inst; i += WAVES) {
         const int e = i * 64 + lane;
-        const uint32_t r = static_cast<uint32_t>(min(e >> shift, a_last));
-        const uint32_t j = static_cast<uint32_t>(min(e & ((1 << shift) - 1), nk - 1));
+        const int row = static_cast<int>((static_cast<float>(e) + 0.5f) * inv_pitch);  // e / pitch, exact for e < 2^20
+        const uint32_t r = static_cast<uint32_t>(min(row, a_last));
+        const uint32_t j = static_cast<uint32_t>(min(e - row * pitch, nk - 1));
         dma_4(reinterpret_cast<const uint8_t*>(as_tile),
               (r * static_cast<uint32_t>(p.as_sm) + j * static_cast<uint32_t>(p.as_sk)) * 4u, smem + Cfg::SCTAB_OFF + i * 256);
       }
@@ -445,6 +449,11 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       wait_vmcnt<0>();
     lds_barrier();
 
+    // first table entry of this lane's rows (scale-table kernels)
+    int tab_row[MF];
+#pragma unroll
+    for (int mi = 0; mi < MF; ++mi) tab_row[mi] = Cfg::SCTAB ? (wm0 + mi * 32 + l32) * p.sct_pitch : 0;
+
     if constexpr (Cfg::PREFETCH) {
       static_assert(kUniformW, "the register-double-buffered path assumes one weight scale per wave");
       // ---- full register double buffering (one wave per SIMD) ------------------------------------------------
@@ -462,7 +471,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
         if constexpr (Cfg::SCTAB) {
           const float* tab = reinterpret_cast<const float*>(smem + Cfg::SCTAB_OFF);
 #pragma unroll
-          for (int mi = 0; mi < MF; ++mi) dst[mi] = tab[((wm0 + mi * 32 + l32) << p.sct_shift) + kbl] * sb;
+          for (int mi = 0; mi < MF; ++mi) dst[mi] = tab[tab_row[mi] + kbl] * sb;
         } else {
           const float* sS = reinterpret_cast<const float*>(smem + base + kScaleOff);
 #pragma unroll
@@ -556,7 +565,7 @@ __device__ __forceinline__ void pipelined_body(const Args& p, uint8_t* smem, int
       const float* tab = reinterpret_cast<const float*>(smem + Cfg::SCTAB_OFF);
 #pragma unroll
       for (int mi = 0; mi < MF; ++mi) {
-        const float sa = Cfg::SCTAB ? tab[((wm0 + mi * 32 + l32) << p.sct_shift) + kbl] : sS[wm0 + mi * 32 + l32];
+        const float sa = Cfg::SCTAB ? tab[tab_row[mi] + kbl] : sS[wm0 + mi * 32 + l32];
 #pragma unroll
         for (int j = 0; j < NS; ++j) dst[mi][j] = sa * sb[j];
       }
