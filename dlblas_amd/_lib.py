@@ -51,7 +51,7 @@ SYMBOLS = {
     'dlb_fp8_gemm_plan': (ctypes.c_int, [ctypes.c_int, _c_i64, _c_i64, _c_i64, _c_sz, ctypes.c_int] + [ctypes.POINTER(ctypes.c_int)] * 3 +
                           [ctypes.POINTER(_c_i64)]),
     'dlb_fp8_gemm_plan_grouped': (ctypes.c_int, [ctypes.c_int, _c_i64, _c_i64, _c_i64, ctypes.c_int32, ctypes.c_int32, _c_sz, ctypes.c_int,
-                                                ctypes.POINTER(ctypes.c_int)]),
+                                                ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
     'dlb_silu_mul': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp] + [_c_i64] * 4 + [_c_vp]),
     'dlb_silu_mul_quant': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp] + [_c_i64] * 5 + [ctypes.c_float, _c_vp]),
     'dlb_silu_mul_quant_masked': (ctypes.c_int, [_c_vp, ctypes.c_int, _c_vp, _c_vp, _c_vp] + [_c_i64] * 6 + [_c_vp]),
@@ -76,6 +76,11 @@ _workspaces = {}
 
 def library_path() -> str:
     return os.environ.get('DLBLAS_AMD_LIB', LIB_PATH)
+
+
+def loaded() -> bool:
+    """Whether load() has already brought the shared library in (never loads it)."""
+    return _lib is not None
 
 
 def load() -> ctypes.CDLL:
@@ -185,12 +190,13 @@ def plan_full(mode: int, rows: int, N: int, K: int, workspace_bytes: int = None,
 
 def plan_grouped(mode: int, rows: int, N: int, K: int, G: int, expected_m: int = -1, workspace_bytes: int = None,
                  compute_units: int = 256):
-    """(variant name,) of a grouped launch (mode 1 contiguous, 2 masked) with G experts and the masked layout's hint."""
+    """(variant name, tile lists used) of a grouped launch (mode 1 contiguous, 2 masked) with G experts and the masked
+    layout's hint; touches no GPU."""
     lib = load()
-    v = ctypes.c_int()
+    v, t = ctypes.c_int(), ctypes.c_int()
     ws = WORKSPACE_BYTES if workspace_bytes is None else workspace_bytes
-    check(lib.dlb_fp8_gemm_plan_grouped(mode, rows, N, K, G, expected_m, ws, compute_units, ctypes.byref(v)))
-    return (variant_names()[v.value], )
+    check(lib.dlb_fp8_gemm_plan_grouped(mode, rows, N, K, G, expected_m, ws, compute_units, ctypes.byref(v), ctypes.byref(t)))
+    return variant_names()[v.value], bool(t.value)
 
 
 def force_variant(name_or_id) -> None:

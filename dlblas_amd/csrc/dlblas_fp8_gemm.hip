@@ -627,11 +627,24 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
   if (mode == kContiguous && pl.variant == kVarPipe128x256w8 && g_forced_variant < 0 && usable_ws && kblocks > 0) {
     const int64_t nblk = ceil_div(rows, kScaleBlock);
     const size_t bytes = tile_list_bytes(nblk);
-    // Taller tiles save weight traffic, not time per tile: while two rounds of 128-row tiles cover the batch, those
-    // are faster and need no list (8 experts, 1408 rows, 4096 x 7168: 107 -> 69 us; 32 experts x 128 rows: 183 ->
-    // 174 us).  The fused epilogues exist for the list kernel only.
-    const bool worth_it = fused_act || gather_scales || g_knob[kKnobTileList] == 1 ||
-                          (g_knob[kKnobTileList] != 2 && nblk * ceil_div(N, 256) > 2ll * cus);
+    // Taller tiles save weight traffic, not time per tile.  Estimates (microseconds, constants as in
+    // prefers_128_row_tiles): uniform 128-row tiles take rounds x (5.5 + K blocks) or, when that is longer, the time
+    // to stream every block's weight matrix (6.4 TB/s: neighbouring tiles of an expert share some of it in the L2);
+    // the lists take 5 us for their pre-pass + rounds x (11.5 + 1.62 K blocks) or the weights of their tiles at
+    // 4.85 TB/s, with as many tiles as pairs of blocks, but at least one per expert.  8 experts, 1408 rows, 4096 x
+    // 7168: 107 us with lists, 69 us without; 2432 rows: 106 us with, 128 us without; 32 experts x 128 rows: 183 / 174.
+    // The fused epilogues exist for the list kernel only.
+    bool worth_it = fused_act || gather_scales || g_knob[kKnobTileList] == 1;
+    if (!worth_it && g_knob[kKnobTileList] != 2 && nblk > G) {
+      const int64_t tn = ceil_div(N, 256);
+      const double mat_mb = static_cast<double>(N) * static_cast<double>(K) * 1e-6;
+      const double plain_us = std::max(static_cast<double>(ceil_div(nblk * tn, cus)) * (5.5 + static_cast<double>(kblocks)),
+                                       static_cast<double>(nblk) * mat_mb / 6.4);
+      const int64_t tall = std::max(ceil_div(nblk, 2), std::min<int64_t>(nblk, G));
+      const double list_us = 5.0 + std::max(static_cast<double>(ceil_div(tall * tn, cus)) * (11.5 + 1.62 * static_cast<double>(kblocks)),
+                                            static_cast<double>(tall) * mat_mb / 4.85);
+      worth_it = list_us < 0.95 * plain_us;
+    }
     if (worth_it && nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
   }
   // Small ring kernels with at most 32 K blocks per workgroup fetch a tile's row-major scales once, into a table in
@@ -1274,7 +1287,7 @@ int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t works
 }
 
 int dlb_fp8_gemm_plan_grouped(int mode, int64_t rows, int64_t N, int64_t K, int32_t G, int32_t expected_m, size_t workspace_bytes,
-                              int compute_units, int* variant) {
+                              int compute_units, int* variant, int* tile_lists) {
   dlb::clear_error();
   if (mode != dlb::kContiguous && mode != dlb::kMasked) return dlb::fail(DLB_ERR_BAD_SHAPE, "mode %d is not 1 (contiguous) or 2 (masked)", mode);
   if (rows < 0 || N < 0 || K < 0 || G < 0) return dlb::fail(DLB_ERR_BAD_SHAPE, "negative dimension (rows=%lld, N=%lld, K=%lld, G=%d)", (long long)rows, (long long)N, (long long)K, G);
@@ -1284,6 +1297,7 @@ int dlb_fp8_gemm_plan_grouped(int mode, int64_t rows, int64_t N, int64_t K, int3
   const dlb::Resolved rs = dlb::resolve(mode, rows, N, K, G, dlb::ceil_div(K, dlb::kScaleBlock), 1, workspace_bytes > 0, workspace_bytes,
                                         compute_units, false, false, mode == dlb::kMasked ? expected_m : -1);
   if (variant) *variant = rs.pl.variant;
+  if (tile_lists) *tile_lists = rs.tile_list ? 1 : 0;
   return DLB_OK;
 }
 

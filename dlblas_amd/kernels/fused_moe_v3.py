@@ -137,8 +137,11 @@ def fused_moe_v3(
     # ep_scatter_rows only fills the tables (which expert and which token each sorted row stands for), the kernel
     # follows them, and neither the expert-sorted copy of the activations nor the bf16 [rows, 2 I] intermediate reaches
     # memory.  Same bits as the steps of the reference (:288-334).
+    # (A batch of at most a round or two of tiles runs faster on uniform 128-row tiles, which have no fused epilogue:
+    # the library's planner says which, and such a batch takes the three steps below.)
     fused = None
-    if tokens_q.is_contiguous() and hidden % 128 == 0 and inter2 % 256 == 0 and n_tokens * hidden < (1 << 32):
+    want_fused = _lib.plan_grouped(1, rows_total, inter2, hidden, w13_weight_fp8[0].size(0))[1]
+    if want_fused and tokens_q.is_contiguous() and hidden % 128 == 0 and inter2 % 256 == 0 and n_tokens * hidden < (1 << 32):
         row_token = buf((rows_total, ), torch.int32)
         ep_scatter_rows(topk_idx, per_expert, first_row, row_expert, row_token, slot_row)
         fused = fp8_gemm_grouped_contiguous_silu_quant(tokens_q, tokens_scale, w13_weight_fp8[0], w13_weight_fp8[1], row_expert,
@@ -153,8 +156,9 @@ def fused_moe_v3(
         sorted_q = buf((rows_total, hidden), torch.uint8).view(tokens_q.dtype)
         sorted_scale = buf((rows_total, hidden // 128), torch.float32)
         ep_scatter(tokens_q, tokens_scale, topk_idx, per_expert, first_row, sorted_q, sorted_scale, row_expert, slot_row)
-        fused = fp8_gemm_grouped_contiguous_silu_quant(sorted_q, sorted_scale, w13_weight_fp8[0], w13_weight_fp8[1], row_expert,
-                                                       column_major_scales=True)
+        if want_fused:
+            fused = fp8_gemm_grouped_contiguous_silu_quant(sorted_q, sorted_scale, w13_weight_fp8[0], w13_weight_fp8[1], row_expert,
+                                                           column_major_scales=True)
         if fused is not None:
             act_q, act_scale = fused
         else:  # the three steps of the reference (:307-334)

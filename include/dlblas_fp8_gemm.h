@@ -313,10 +313,14 @@ int dlb_fp8_gemm_plan(int mode, int64_t rows, int64_t N, int64_t K, size_t works
 /*
  * The same query for the grouped layouts with what their choice depends on besides the shape: the expert count and, for
  * the masked layout (mode 2), the caller's expected_m (<= 0: unknown).  mode 1 = contiguous (rows = M_sum), 2 = masked
- * (rows = M_max).  No counterpart in the reference.
+ * (rows = M_max).  Outputs (each may be NULL): the kernel variant id; whether a contiguous launch of this size pairs
+ * blocks into taller tiles from lists built on the device (1) or runs uniform 128-row tiles (0).  The fused gate/up
+ * entry points always take the lists, so a caller that can also run GEMM and activation apart does that where this
+ * says 0 (a batch of at most a round or two of tiles, where the uniform tiles are faster).  No counterpart in the
+ * reference.
  */
 int dlb_fp8_gemm_plan_grouped(int mode, int64_t rows, int64_t N, int64_t K, int32_t G, int32_t expected_m, size_t workspace_bytes,
-                              int compute_units, int* variant);
+                              int compute_units, int* variant, int* tile_lists);
 
 /*
  * Tuning / test hook: force the kernel variant the next calls FROM THIS THREAD use.

@@ -22,6 +22,17 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+@pytest.fixture(autouse=True)
+def _library_heuristics_restored():
+    """A test that pins a kernel variant or sets a tuning knob and then fails must not change what later tests run."""
+    yield
+    from dlblas_amd import _lib
+    if _lib.loaded():
+        _lib.force_variant(None)
+        for knob in _lib.KNOBS:
+            _lib.tune(knob, 0)
+
+
 def pytest_terminal_summary(terminalreporter):
     """Relative error at the strict floor (|ref| floored at 1e-3 rms) of every parity check that ran: reported, not
     asserted (the asserted bars are in helpers.tolerance_check)."""

@@ -186,13 +186,19 @@ def test_tma_align_input_scale(dev):
     assert torch.equal(tma_align_input_scale(s.to(dev)).cpu(), s)
 
 
-def test_fused_moe_v3_end_to_end(dev):
+@pytest.mark.parametrize('tile_lists', [0, 1])
+def test_fused_moe_v3_end_to_end(dev, tile_lists):
     """scatter -> GEMM -> silu*up + quant -> GEMM -> gather against the same chain of oracles.  The device's GEMM
     differs from the oracle's within the GEMM tolerance, which the quantiser between the GEMMs can turn into a
     different fp8 code here and there; the bar is the reference's similarity metric plus a bound on the largest
-    deviation relative to the output's rms."""
+    deviation relative to the output's rms.  A batch this small takes the three steps of the reference on uniform
+    tiles (tile_lists = 0: the library's choice); with the tile lists forced it takes the fused gate/up kernel that
+    reads the tokens where they lie, as large batches do."""
+    from dlblas_amd import _lib
     from dlblas_amd.kernels.fused_moe_v3 import fused_moe_v3
-    print('case fused_moe_v3', flush=True)
+    print(f'case fused_moe_v3 tile_lists={tile_lists}', flush=True)
+    _lib.tune('tile_list', tile_lists)
+    assert _lib.plan_grouped(1, 512, 1024, 512, 4)[1] == bool(tile_lists)
     T, K, N, E, topk = 96, 512, 1024, 4, 2  # N = gate + up
     g = helpers.gen(77)
     x = torch.randn(T, K, generator=g).to(torch.bfloat16)
@@ -233,6 +239,7 @@ def test_fused_moe_v3_end_to_end(dev):
     # the two early exits of the reference driver (fused_moe_v3.py:255-259)
     assert torch.equal(fused_moe_v3((x_q.to(dev), x_s.to(dev)), ids.to(dev), wts.to(dev), None, None, None).cpu(),
                        x_q.to(torch.bfloat16))
+    _lib.tune('tile_list', 0)
 
 
 def test_fused_moe_v3_full_size_sampled_tokens(dev):
