@@ -179,14 +179,18 @@ def test_activation_argument_validation(dev):
         silu_and_mul_post_quant(torch.zeros(4, 200, dtype=torch.bfloat16, device=dev))
 
 
-def test_low_latency_experts_end_to_end(dev):
+@pytest.mark.parametrize('expected_m', [32, 0])
+def test_low_latency_experts_end_to_end(dev, expected_m):
     """masked GEMM -> masked silu*up + quant -> masked GEMM (dlblas/layers/moe/ep_moe.py:199-261) against the same
     chain of oracles on the valid rows.  Bar as for the contiguous driver: the reference's similarity metric plus a
     bound on the largest deviation relative to the output's rms (the quantiser between the GEMMs can turn a GEMM
     difference within tolerance into a different fp8 code)."""
+    from dlblas_amd import _lib
     from dlblas_amd.kernels.moe import low_latency_experts
-    print('case low_latency_experts', flush=True)
+    print(f'case low_latency_experts expected_m={expected_m}', flush=True)
     G, M, K, N = 4, 48, 512, 1024
+    # a few short experts get 128 x 128 tiles and the steps apart; without the hint the fused gate/up kernel runs
+    assert _lib.plan_grouped(2, M, N, K, G, expected_m)[0] == ('pipe128x128' if expected_m > 0 else 'pipe128x256w8')
     g = helpers.gen(91)
     masked = torch.tensor([0, 48, 17, 33], dtype=torch.int32)
     a_q, a_s = orc.quant_act_1x128(torch.randn(G, M, K, generator=g).to(torch.bfloat16))
@@ -198,7 +202,7 @@ def test_low_latency_experts_end_to_end(dev):
         w2.append(q), w2_s.append(s)
     w13, w13_s, w2, w2_s = torch.stack(w13), torch.stack(w13_s), torch.stack(w2), torch.stack(w2_s)
     out = low_latency_experts((a_q.to(dev), a_s.to(dev)), w13.to(dev), w13_s.to(dev), w2.to(dev), w2_s.to(dev),
-                              masked.to(dev), 32)
+                              masked.to(dev), expected_m)
     torch.cuda.synchronize()
     gateup = torch.zeros(G, M, N, dtype=torch.bfloat16)
     orc.grouped_masked_ref(a_q, a_s, w13, w13_s, gateup, masked)
