@@ -555,14 +555,17 @@ Plan make_plan(int mode, int64_t M, int64_t N, int64_t K, int cus, size_t ws_byt
   if (is_skinny(v)) {
     // K is split over the waves of a workgroup only.  Pick the wave count so that every wave has two or so K
     // blocks and the unroll so that a wave issues all of its loads before its first MFMA.
-    int waves = kblocks >= 8 ? 8 : 4;
+    int waves = kblocks >= 4 ? 8 : 4;  // (4 K blocks: 16 x 32768 x 512 7.4 -> 6.4 us with 8 waves, half of them without a block)
     // A long K against few rows: 16 waves keep twice the weight bytes in flight (1 x 2112 x 7168: 7.3 -> 6.0 us) - as
     // long as the workgroup's share of the weights is small (up to 16 rows of K = 7168: 16 x 4096 x 7168 8.4 -> 8.2 us,
     // 16 x 1536 x 7168 7.6 -> 6.4 us; from 20 rows on 8 waves are ahead: 16 x 7168 x 16384 21.7 -> 20.5 us) and one
     // round of workgroups covers the matrix (16 x 36864 x 7168: 55 -> 47 us with 8 waves).
-    if (skinny_rows(v) == 16 && kblocks >= 48 && K % kScaleBlock == 0) {
+    // (from 24 K blocks on for up to 8 rows: 1 x 4096 x 4096 6.0 -> 5.25 us, 1 x 3072 x 3072 4.9 -> 4.4 us)
+    if (skinny_rows(v) == 16 && kblocks >= (M <= 8 ? 24 : 48) && K % kScaleBlock == 0) {
       const int bn16 = g_knob[kKnobSkinnyBn] > 0 ? g_knob[kKnobSkinnyBn] : pick_skinny_bn(N, 16, cus);
-      if (static_cast<int64_t>(bn16) * K <= 128 * 1024 && ceil_div(N, bn16) <= cus) waves = 16;
+      // (a single row moves the limit up: 1 x 4608 x 7168, 20 rows of K = 7168 per workgroup, 9.4 -> 8.5 us with 16 waves)
+      const int64_t share_limit = (M <= 8 ? 160 : 128) * 1024;
+      if (static_cast<int64_t>(bn16) * K <= share_limit && ceil_div(N, bn16) <= cus) waves = 16;
     }
     if (g_knob[kKnobSkinnyWaves] > 0) waves = g_knob[kKnobSkinnyWaves] >= 16 ? 16 : (g_knob[kKnobSkinnyWaves] >= 8 ? 8 : 4);
     const int per_wave = static_cast<int>(ceil_div(kblocks, waves));

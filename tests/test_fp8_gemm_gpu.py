@@ -36,6 +36,7 @@ DENSE_SHAPES = [
     (512, 512, 512),      # the shape of tests/kernels/test_fp8_gemm.py
     (1, 7168, 2048), (16, 7168, 2048), (64, 7168, 2048), (128, 7168, 2048),
     (1, 2112, 7168), (16, 2112, 7168), (64, 2112, 7168), (128, 2112, 7168),
+    (16, 1000, 640), (1, 392, 896), (32, 520, 512),  # decode with 4 to 7 K blocks: 8 waves, some of them without a block
     (300, 2112, 1536),    # ragged M and N tiles
     (256, 7168, 2048), (384, 2112, 7168), (130, 7168, 16384),  # between decode and prefill: small tiles, K split over workgroups
     (129, 130, 384),      # N not a multiple of 4: scalar stores
