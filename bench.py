@@ -701,6 +701,169 @@ def copy_calibration(dev):
     del src, dst
 
 
+PLANNER_SWEEP_WEIGHTS = [(2112, 7168), (24576, 1536), (32768, 512), (7168, 16384), (4096, 7168), (7168, 2048), (1536, 7168),
+                         (7168, 18432), (36864, 7168), (576, 7168), (4608, 7168), (7168, 2304), (18432, 7168)]
+
+
+def planner_sweep(dev, which):
+    """The planner's launch against every alternative forced in turn; prints one line per problem and returns the rows.
+    'dense': kernel variants (no K split forced) over 13 weight shapes x 15 row counts; 'mid': the three small ring
+    kernels x 1 ... 16 K slices where the planner picks one of them; 'decode': columns per workgroup x waves x blocks in
+    flight of the streaming kernels at 1, 16 and 32 rows; 'grouped': ring variants for both grouped layouts, 8 and 32
+    experts.  A row's 'regret' is default / best - 1."""
+    import torch
+
+    from dlblas_amd import _lib
+    from dlblas_amd.kernels.fp8_gemm_grouped import fp8_gemm_grouped_contiguous, fp8_gemm_grouped_masked
+    rows = []
+
+    def report(name, plan, t_default, best_t, best_what):
+        row = {'problem': name, 'plan': plan, 'default_us': t_default, 'best_us': best_t, 'best': best_what,
+               'regret': t_default / best_t - 1.0}
+        rows.append(row)
+        print(f"{name}: default {plan} {t_default:.1f} us; best {best_what} {best_t:.1f} us; regret {100 * row['regret']:.0f} %", flush=True)
+
+    def dense_problem(M, N, K):
+        copies = max(2, min(24, int(400e6 // (N * K))))
+        a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=copies)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        launch = DenseLauncher(a_q, a_s, ws, out)
+        reps = int(max(10, min(200, 3e-2 / max(2.0 * M * N * K / 2e15, 5e-6))))
+        time_call(launch, reps, reps)
+        return launch, reps
+
+    def timed(launch, reps):
+        try:
+            launch()
+            torch.cuda.synchronize()
+            return time_call(launch, reps, max(5, reps // 4)) * 1e3
+        except Exception:  # the variant does not take this shape
+            return None
+
+    try:
+        if which == 'dense':
+            names = [n for n in _lib.variant_names() if n.startswith('pipe') or n.startswith('skinny')]
+            for (N, K) in PLANNER_SWEEP_WEIGHTS:
+                for M in (1, 16, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 2048, 4096):
+                    if M * N * K > 4096 * 7168 * 18432:
+                        continue
+                    launch, reps = dense_problem(M, N, K)
+                    plan = _lib.plan(0, M, N, K)
+                    t0 = timed(launch, reps)
+                    best = (t0, 'default')
+                    if plan[1] == 1:  # forcing a variant drops the K split the planner chose with it
+                        for v in names:
+                            _lib.force_variant(v)
+                            t = timed(launch, reps)
+                            if t is not None and t < best[0]:
+                                best = (t, v)
+                        _lib.force_variant(None)
+                        t0 = min(t0, timed(launch, reps))
+                    report(f'{M}x{N}x{K}', plan[:2], t0, min(best[0], t0), best[1])
+        elif which == 'mid':
+            for (N, K) in PLANNER_SWEEP_WEIGHTS + [(4096, 4096), (1024, 16384), (7168, 4096)]:
+                for M in (48, 64, 96, 128, 192, 256, 384, 512, 1024):
+                    plan = _lib.plan(0, M, N, K)
+                    if plan[0] not in ('pipe128x256w8', 'pipe128x128', 'pipe128x64') or M * N * K > 4096 * 7168 * 4096:
+                        continue
+                    launch, reps = dense_problem(M, N, K)
+                    t0 = timed(launch, reps)
+                    best = (t0, 'default')
+                    for v in ('pipe128x256w8', 'pipe128x128', 'pipe128x64'):
+                        _lib.force_variant(v)
+                        for sk in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16):
+                            if sk > 1 and (K // 128) // sk < 2:
+                                continue
+                            _lib.tune('splitk', sk)
+                            t = timed(launch, max(10, reps // 2))
+                            if t is not None and t < best[0]:
+                                best = (t, f'{v} / {sk} slices')
+                        _lib.tune('splitk', 0)
+                    _lib.force_variant(None)
+                    t0 = min(t0, timed(launch, reps))
+                    report(f'{M}x{N}x{K}', plan[:2], t0, min(best[0], t0), best[1])
+        elif which == 'decode':
+            for (N, K) in PLANNER_SWEEP_WEIGHTS + [(4096, 4096), (8192, 1024), (16384, 2048)]:
+                for M in (1, 16, 32):
+                    launch, reps = dense_problem(M, N, K)
+                    plan = _lib.plan(0, M, N, K)
+                    t0 = timed(launch, reps)
+                    best = (t0, 'default')
+                    for bn in (8, 12, 16, 20, 24, 28, 32):
+                        for waves in (4, 8, 16):
+                            for unroll in (1, 2):
+                                _lib.tune('skinny_bn', bn), _lib.tune('skinny_waves', waves), _lib.tune('skinny_unroll', unroll)
+                                t = timed(launch, max(10, reps // 2))
+                                if t is not None and t < best[0]:
+                                    best = (t, f'{bn} columns, {waves} waves, {unroll} in flight')
+                    for knob in ('skinny_bn', 'skinny_waves', 'skinny_unroll'):
+                        _lib.tune(knob, 0)
+                    t0 = min(t0, timed(launch, reps))
+                    report(f'{M}x{N}x{K}', plan, t0, min(best[0], t0), best[1])
+        elif which == 'grouped':
+            gd = torch.Generator(device=dev).manual_seed(21)
+            ring = ('pipe128x256w8', 'pipe256x256', 'pipe128x128')
+            for (G, N, K) in ((32, 4096, 7168), (32, 7168, 2048), (8, 4096, 7168), (8, 7168, 2048)):
+                w_q, w_s = expert_weights(G, N, K, dev, 22)
+                for tokens in (G * 16, G * 64, G * 128, G * 256, G * 512):
+                    assign = torch.multinomial(torch.full((G, ), 1.0 / G), tokens, replacement=True,
+                                               generator=torch.Generator().manual_seed(20))
+                    padded = (torch.bincount(assign, minlength=G) + 127) // 128 * 128
+                    M_sum = int(padded.sum())
+                    m_indices = torch.repeat_interleave(torch.arange(G, dtype=torch.int32), padded).to(dev)
+                    a_q, a_s = quantise_act(torch.randn(M_sum, K, device=dev, generator=gd).to(torch.bfloat16))
+                    out = torch.empty(M_sum, N, dtype=torch.bfloat16, device=dev)
+                    call = lambda: fp8_gemm_grouped_contiguous(a_q, a_s, w_q, w_s, out, m_indices)  # noqa: E731
+                    t0 = timed(call, 30)
+                    best = (t0, 'default')
+                    for v in ring:
+                        _lib.force_variant(v)
+                        t = timed(call, 30)
+                        if t is not None and t < best[0]:
+                            best = (t, v + ', uniform tiles')
+                    _lib.force_variant(None)
+                    for lists in (1, 2):
+                        _lib.tune('tile_list', lists)
+                        t = timed(call, 30)
+                        if t is not None and t < best[0]:
+                            best = (t, 'tile lists' if lists == 1 else 'no tile lists')
+                    _lib.tune('tile_list', 0)
+                    t0 = min(t0, timed(call, 30))
+                    report(f'contiguous, {G} experts, {M_sum} rows, {N}x{K}', _lib.plan_grouped(1, M_sum, N, K, G), t0, min(best[0], t0), best[1])
+                    del a_q, a_s, out
+                for M_max in (64, 128, 256, 512, 1024):
+                    for fill in (0.1, 0.5, 1.0):
+                        masked_m = torch.randint(0, int(M_max * fill) + 1, (G, ), generator=torch.Generator().manual_seed(20), dtype=torch.int32)
+                        a_q, a_s = quantise_act(torch.randn(G * M_max, K, device=dev, generator=gd).to(torch.bfloat16))
+                        a_q, a_s = a_q.reshape(G, M_max, K), a_s.reshape(G, M_max, K // 128)
+                        out = torch.empty(G, M_max, N, dtype=torch.bfloat16, device=dev)
+                        mm, hint = masked_m.to(dev), int(masked_m.float().mean())
+                        call = lambda: fp8_gemm_grouped_masked(a_q, a_s, w_q, w_s, out, mm, hint)  # noqa: E731
+                        t0 = timed(call, 30)
+                        best = (t0, 'default')
+                        for v in ring:
+                            _lib.force_variant(v)
+                            t = timed(call, 30)
+                            if t is not None and t < best[0]:
+                                best = (t, v)
+                        _lib.force_variant(None)
+                        t0 = min(t0, timed(call, 30))
+                        report(f'masked, {G} experts x {M_max} slots, {int(masked_m.sum())} valid rows, {N}x{K}',
+                               _lib.plan_grouped(2, M_max, N, K, G, hint), t0, min(best[0], t0), best[1])
+                        del a_q, a_s, out
+                del w_q, w_s
+        else:
+            raise ValueError(which)
+    finally:
+        _lib.force_variant(None)
+        for knob in _lib.KNOBS:
+            _lib.tune(knob, 0)
+    worst = sorted(rows, key=lambda r: -r['regret'])[:5]
+    print(f"{len(rows)} problems; over 5 %: {sum(r['regret'] > 0.05 for r in rows)}, over 10 %: {sum(r['regret'] > 0.10 for r in rows)}; "
+          'largest: ' + '; '.join(f"{r['problem']} {100 * r['regret']:.0f} %" for r in worst), flush=True)
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -726,6 +889,9 @@ def main():
     ap.add_argument('--grouped-only', action='store_true',
                     help='run only the two grouped MoE workloads and print their rows (the command the rocprofv3 summaries of '
                     'the grouped kernels are made with)')
+    ap.add_argument('--planner-sweep', choices=['dense', 'mid', 'decode', 'grouped'], default=None,
+                    help="time the planner's launch against every alternative forced in turn over a grid of problems and "
+                    'print where it is not the fastest (a minute or two)')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1', file=sys.stderr)
@@ -743,6 +909,10 @@ def main():
 
     if args.decode_floor:
         print(json.dumps({'decode_floor': decode_floor(dev)}), flush=True)
+        return
+
+    if args.planner_sweep:
+        planner_sweep(dev, args.planner_sweep)
         return
 
     if args.ceilings:

@@ -631,7 +631,7 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
     const int64_t nblk = ceil_div(rows, kScaleBlock);
     const size_t bytes = tile_list_bytes(nblk);
     // Taller tiles save weight traffic, not time per tile.  Estimates (microseconds, constants as in
-    // prefers_128_row_tiles): uniform 128-row tiles take rounds x (5.5 + K blocks) or, when that is longer, the time
+    // prefers_128_row_tiles): uniform 128-row tiles take rounds x (5.5 + 1.2 K blocks: most of their weights come from HBM) or, when that is longer, the time
     // to stream every block's weight matrix (6.4 TB/s: neighbouring tiles of an expert share some of it in the L2);
     // the lists take 5 us for their pre-pass + rounds x (11.5 + 1.62 K blocks) or the weights of their tiles at
     // 4.85 TB/s, with as many tiles as pairs of blocks, but at least one per expert.  8 experts, 1408 rows, 4096 x
@@ -641,12 +641,12 @@ Resolved resolve(int mode, int64_t rows, int64_t N, int64_t K, int G, int64_t as
     if (!worth_it && g_knob[kKnobTileList] != 2 && nblk > G) {
       const int64_t tn = ceil_div(N, 256);
       const double mat_mb = static_cast<double>(N) * static_cast<double>(K) * 1e-6;
-      const double plain_us = std::max(static_cast<double>(ceil_div(nblk * tn, cus)) * (5.5 + static_cast<double>(kblocks)),
+      const double plain_us = std::max(static_cast<double>(ceil_div(nblk * tn, cus)) * (5.5 + 1.2 * static_cast<double>(kblocks)),
                                        static_cast<double>(nblk) * mat_mb / 6.4);
       const int64_t tall = std::max(ceil_div(nblk, 2), std::min<int64_t>(nblk, G));
       const double list_us = 5.0 + std::max(static_cast<double>(ceil_div(tall * tn, cus)) * (11.5 + 1.62 * static_cast<double>(kblocks)),
                                             static_cast<double>(tall) * mat_mb / 4.85);
-      worth_it = list_us < 0.95 * plain_us;
+      worth_it = list_us < plain_us;
     }
     if (worth_it && nblk <= kTileListMaxBlocks && DLB_WS_COUNTER_BYTES + bytes <= ws_bytes) r.tile_list = true, r.nblk = nblk, r.ws_used = bytes;
   }
