@@ -259,6 +259,8 @@ def decode_floor(dev, N=7168, K=2048, copies=24):
     lib = ctypes.CDLL(FLOOR_LIB)
     lib.floor_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
     lib.floor_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.floor_read_store.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64,
+                                     ctypes.c_void_p]
     bufs = [torch.randint(0, 255, (N * K, ), dtype=torch.uint8, device=dev) for _ in range(copies)]
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
@@ -279,11 +281,30 @@ def decode_floor(dev, N=7168, K=2048, copies=24):
             tried[f'{per_cu} wg/cu x {depth} loads'] = time_call(reader(cus * per_cu, depth), 240, 240) * 1e3
     best = min(tried, key=tried.get)
     read_us = time_call(reader(cus * int(best.split()[0]), int(best.split()[3])), 480, 1500) * 1e3
+    # the same reads + one exchange between a workgroup's waves + the store of a 16-row bf16 result (fastest shape again)
+    out16 = torch.empty(16 * N, dtype=torch.bfloat16, device=dev)
+
+    def storer(wgs, depth):
+        def run():
+            b = bufs[state['i']]
+            state['i'] = (state['i'] + 1) % copies
+            lib.floor_read_store(ctypes.c_void_p(b.data_ptr()), N * K, wgs, depth, ctypes.c_void_p(out16.data_ptr()), out16.numel() * 2, stream)
+        return run
+
+    tried_store = {}
+    for per_cu in (1, 2, 4):
+        for depth in (2, 4, 8):
+            tried_store[f'{per_cu} wg/cu x {depth} loads'] = time_call(storer(cus * per_cu, depth), 240, 240) * 1e3
+    best_store = min(tried_store, key=tried_store.get)
+    read_store_us = time_call(storer(cus * int(best_store.split()[0]), int(best_store.split()[3])), 480, 1500) * 1e3
     del bufs
     return {'empty_launch_us': empty_ms * 1e3, 'read_only_us': read_us, 'read_only_GBps': N * K / read_us / 1e3,
+            'read_exchange_store_us': read_store_us, 'read_exchange_store_shape': best_store,
+            'gemm_16_rows_us': decode_stream_loop(dev, 16, N, K, copies),
             'read_only_shape': best, 'bytes_read': N * K, 'gemm_16_rows_graph_replay_us': decode_graph_replay(dev, 16, N, K, copies),
             'note': 'bench-only kernels (bench_kernels/floor_kernels.hip), same rotation of weight buffers and same launch '
                     'loop as the decode rows; read_only = fastest of 9 shapes of a kernel that only loads the weight bytes; '
+                    'read_exchange_store = the same reads, one LDS exchange between the waves of a workgroup and the store of a 16-row bf16 result; '
                     'graph_replay = the GEMM itself, 48 launches captured in a HIP graph and replayed'}
 
 
@@ -316,6 +337,14 @@ def decode_graph_replay(dev, M, N, K, copies):
         side.synchronize()
     torch.cuda.current_stream().wait_stream(side)
     return start.elapsed_time(stop) / (10 * per_graph) * 1e3
+
+
+def decode_stream_loop(dev, M, N, K, copies):
+    """Per-launch time of the decode GEMM in the loop the floors are measured in (launches back to back on one stream)."""
+    import torch
+    a_q, a_s, ws = make_inputs(M, N, K, dev, weight_copies=copies)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    return time_call(DenseLauncher(a_q, a_s, ws, out), 480, 1500) * 1e3
 
 
 def ceilings(dev):

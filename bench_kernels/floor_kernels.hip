@@ -46,6 +46,29 @@ __global__ void __launch_bounds__(512) floor_read_kernel(const v4i* src, int64_t
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5a5a5a5a && sink == reinterpret_cast<int*>(1)) *sink = acc.x;
 }
 
+// The same reads, then what any GEMM of that shape also has to do at its end: one exchange between the waves of a
+// workgroup through LDS (a barrier) and the store of the workgroup's share of `out_bytes` of output.
+template <int U>
+__global__ void __launch_bounds__(512) floor_read_store_kernel(const v4i* src, int64_t words, int* out, int64_t out_bytes) {
+  __shared__ int xch[512];
+  v4i acc = {0, 0, 0, 0};
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  for (; i + (U - 1) * stride < words; i += U * stride) {
+    v4i v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u];
+  }
+  for (; i < words; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+  xch[threadIdx.x] = acc.x ^ acc.y ^ acc.z ^ acc.w;
+  __syncthreads();
+  const int mixed = xch[threadIdx.x] ^ xch[(threadIdx.x + 64) & 511] ^ xch[(threadIdx.x + 192) & 511];
+  const int64_t per_wg = out_bytes / 4 / gridDim.x;  // dwords of output per workgroup
+  for (int64_t t = threadIdx.x; t < per_wg; t += 512) out[static_cast<int64_t>(blockIdx.x) * per_wg + t] = mixed;
+}
+
 // R = ds_read_b128 per MFMA pair (0 or 3).  in: 6 x 64 x 32 bytes of e4m3 codes (4 "A" + 2 "B" operand registers per lane).
 template <int R>
 __global__ void __launch_bounds__(512) floor_mfma_kernel(const v8i* in, float* out, int iters, float scale) {
@@ -199,6 +222,20 @@ int floor_read(const void* src, int64_t bytes, int workgroups, int loads_in_flig
     hipLaunchKernelGGL(floor_read_kernel<4>, grid, block, 0, st, p, bytes / 16, nullptr);
   else
     hipLaunchKernelGGL(floor_read_kernel<2>, grid, block, 0, st, p, bytes / 16, nullptr);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int floor_read_store(const void* src, int64_t bytes, int workgroups, int loads_in_flight, void* out, int64_t out_bytes, void* stream) {
+  const dim3 grid(workgroups), block(512);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const v4i* p = static_cast<const v4i*>(src);
+  int* o = static_cast<int*>(out);
+  if (loads_in_flight >= 8)
+    hipLaunchKernelGGL(floor_read_store_kernel<8>, grid, block, 0, st, p, bytes / 16, o, out_bytes);
+  else if (loads_in_flight >= 4)
+    hipLaunchKernelGGL(floor_read_store_kernel<4>, grid, block, 0, st, p, bytes / 16, o, out_bytes);
+  else
+    hipLaunchKernelGGL(floor_read_store_kernel<2>, grid, block, 0, st, p, bytes / 16, o, out_bytes);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
