@@ -49,6 +49,32 @@ def test_prefill_full_size(dev, M, N, K):
     assert torch.equal(out3, out[perm])
 
 
+@pytest.mark.parametrize('M,N,K,variant,slices', [
+    (384, 18432, 7168, 'pipe128x256w8', 1),    # two 256-row tiles would be half padding: three rows of 128 x 256 tiles
+    (2048, 4096, 7168, 'pipe128x256w8', 1),    # 128 tiles of 256 x 256 would leave half the CUs idle
+    (4096, 32768, 512, 'pipe128x256w8', 1),    # four K blocks: 16 rounds of resident workgroups
+    (512, 4096, 7168, 'pipe128x64', 1),        # the scale table at 56 K blocks
+    (64, 1024, 16384, 'pipe128x64', 16),       # 16 K slices
+    (16, 36864, 7168, 'skinny16', 1),          # six rounds of decode workgroups
+])
+def test_planner_choices_full_size(dev, M, N, K, variant, slices):
+    """Shapes whose launch the planner's later rules decide, at their real size: sampled rows against the oracle,
+    exact power-of-two linearity, row permutation."""
+    from dlblas_amd import _lib
+    print(f'case planner choice full size M={M} N={N} K={K}', flush=True)
+    assert _lib.plan(0, M, N, K)[:2] == (variant, slices)
+    a_q, a_s, b_q, b_s = helpers.make_dense_device(M, N, K, dev, seed=M + K)
+    out = _gemm(a_q, b_q, a_s, b_s)
+    torch.cuda.synchronize()
+    rows = _sample_rows(M, min(M, 24), 3)
+    ref = orc.dequant_ref(a_q[rows].cpu(), a_s[rows].cpu(), b_q.cpu(), b_s.cpu())
+    helpers.tolerance_check(out[rows], ref, f'planner choice {M}x{N}x{K} sampled rows')
+    assert torch.equal(_gemm(a_q, b_q, a_s * 4, b_s), out * 4)
+    if variant != 'skinny16':  # (the decode kernels' summation order depends on the row fragment a row falls into)
+        perm = torch.randperm(M, generator=torch.Generator().manual_seed(4)).to(dev)
+        assert torch.equal(_gemm(a_q[perm].contiguous(), b_q, a_s[perm].contiguous(), b_s), out[perm])
+
+
 @pytest.mark.parametrize('M', [1, 16, 64, 128])
 @pytest.mark.parametrize('N,K', [(7168, 2048), (2112, 7168)])
 def test_decode_full_size(dev, M, N, K):
